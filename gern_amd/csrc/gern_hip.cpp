@@ -1,0 +1,434 @@
+// Implementation of the C ABI declared in include/gern_hip.h: hiprtc compile,
+// hipModule load, kernel lookup by name expression, checked launch, memory and
+// event helpers.  Host code only; it links libamdhip64 and libhiprtc.
+#include "gern_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string &msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    return fail(GERN_HIP_ERR_RUNTIME, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(call)                           \
+    do {                                        \
+        hipError_t e_ = (call);                 \
+        if (e_ != hipSuccess) {                 \
+            return hip_fail(e_, #call);         \
+        }                                       \
+    } while (0)
+
+std::mutex g_limits_mutex;
+bool g_limits_ready = false;
+gern_hip_limits g_limits;
+
+int load_limits() {
+    std::lock_guard<std::mutex> lock(g_limits_mutex);
+    if (g_limits_ready) {
+        return GERN_HIP_OK;
+    }
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) {
+        return fail(GERN_HIP_ERR_NO_DEVICE, "no HIP device is visible to this process");
+    }
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, 0));
+    std::memset(&g_limits, 0, sizeof(g_limits));
+    g_limits.wavefront_size = prop.warpSize;
+    g_limits.max_threads_per_block = prop.maxThreadsPerBlock;
+    for (int i = 0; i < 3; i++) {
+        g_limits.max_block_dim[i] = prop.maxThreadsDim[i];
+        g_limits.max_grid_dim[i] = prop.maxGridSize[i];
+    }
+    g_limits.lds_bytes_per_block = (int64_t)prop.sharedMemPerBlock;
+    int optin = 0;
+    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, 0) == hipSuccess &&
+        optin > g_limits.lds_bytes_per_block) {
+        g_limits.lds_bytes_per_block = optin;
+    }
+    g_limits.compute_units = prop.multiProcessorCount;
+    g_limits.clock_khz = prop.clockRate;
+    g_limits.hbm_bytes = (int64_t)prop.totalGlobalMem;
+    std::snprintf(g_limits.arch, sizeof(g_limits.arch), "%s", prop.gcnArchName);
+    g_limits_ready = true;
+    return GERN_HIP_OK;
+}
+
+struct CompiledProgram {
+    std::vector<char> code;
+    std::map<std::string, std::string> lowered;  // name expression -> mangled name
+};
+
+int compile_program(const char *source, const char *const *name_exprs, int n_name_exprs,
+                    const char *const *options, int n_options, const char *arch,
+                    CompiledProgram &out) {
+    if (source == nullptr || (n_name_exprs > 0 && name_exprs == nullptr) ||
+        (n_options > 0 && options == nullptr)) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_compile: null argument");
+    }
+    std::string arch_name = arch ? arch : "";
+    if (arch_name.empty()) {
+        int rc = load_limits();
+        if (rc != GERN_HIP_OK) {
+            return rc;
+        }
+        arch_name = g_limits.arch;
+    }
+    hiprtcProgram prog;
+    hiprtcResult r = hiprtcCreateProgram(&prog, source, "gern_generated.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS) {
+        return fail(GERN_HIP_ERR_COMPILE, std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+    }
+    for (int i = 0; i < n_name_exprs; i++) {
+        r = hiprtcAddNameExpression(prog, name_exprs[i]);
+        if (r != HIPRTC_SUCCESS) {
+            hiprtcDestroyProgram(&prog);
+            return fail(GERN_HIP_ERR_COMPILE, std::string("hiprtcAddNameExpression(") + name_exprs[i] +
+                                                  "): " + hiprtcGetErrorString(r));
+        }
+    }
+    std::vector<std::string> opt_storage;
+    opt_storage.push_back("--offload-arch=" + arch_name);
+    opt_storage.push_back("-O3");
+    opt_storage.push_back("-std=c++17");
+    // Packed-FP32 instructions are kept out of every kernel.
+    opt_storage.push_back("-Xclang");
+    opt_storage.push_back("-target-feature");
+    opt_storage.push_back("-Xclang");
+    opt_storage.push_back("-packed-fp32-ops");
+    for (int i = 0; i < n_options; i++) {
+        opt_storage.push_back(options[i]);
+    }
+    std::vector<const char *> opts;
+    for (const auto &o : opt_storage) {
+        opts.push_back(o.c_str());
+    }
+    r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
+    if (r != HIPRTC_SUCCESS) {
+        size_t log_size = 0;
+        hiprtcGetProgramLogSize(prog, &log_size);
+        std::string log(log_size, '\0');
+        if (log_size > 0) {
+            hiprtcGetProgramLog(prog, log.data());
+        }
+        hiprtcDestroyProgram(&prog);
+        return fail(GERN_HIP_ERR_COMPILE, std::string("hiprtc: ") + hiprtcGetErrorString(r) + "\n" + log);
+    }
+    for (int i = 0; i < n_name_exprs; i++) {
+        const char *lowered = nullptr;
+        r = hiprtcGetLoweredName(prog, name_exprs[i], &lowered);
+        if (r != HIPRTC_SUCCESS || lowered == nullptr) {
+            hiprtcDestroyProgram(&prog);
+            return fail(GERN_HIP_ERR_COMPILE, std::string("no kernel matches name expression ") + name_exprs[i]);
+        }
+        out.lowered[name_exprs[i]] = lowered;
+    }
+    size_t code_size = 0;
+    r = hiprtcGetCodeSize(prog, &code_size);
+    if (r != HIPRTC_SUCCESS || code_size == 0) {
+        hiprtcDestroyProgram(&prog);
+        return fail(GERN_HIP_ERR_COMPILE, "hiprtc produced no code object");
+    }
+    out.code.resize(code_size);
+    hiprtcGetCode(prog, out.code.data());
+    hiprtcDestroyProgram(&prog);
+    return GERN_HIP_OK;
+}
+
+}  // namespace
+
+struct gern_hip_module_s {
+    hipModule_t module = nullptr;
+    std::map<std::string, std::string> lowered;
+    std::vector<gern_hip_kernel_s *> kernels;
+};
+
+struct gern_hip_kernel_s {
+    hipFunction_t fn = nullptr;
+    std::string name;
+};
+
+struct gern_hip_event_s {
+    hipEvent_t ev = nullptr;
+};
+
+extern "C" {
+
+int gern_hip_compile(const char *source, const char *const *name_exprs, int n_name_exprs,
+                     const char *const *options, int n_options, const char *arch,
+                     gern_hip_module *out) {
+    if (out == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_compile: null output handle");
+    }
+    *out = nullptr;
+    int rc = load_limits();
+    if (rc != GERN_HIP_OK) {
+        return rc;
+    }
+    CompiledProgram prog;
+    rc = compile_program(source, name_exprs, n_name_exprs, options, n_options, arch, prog);
+    if (rc != GERN_HIP_OK) {
+        return rc;
+    }
+    auto *m = new gern_hip_module_s();
+    hipError_t e = hipModuleLoadData(&m->module, prog.code.data());
+    if (e != hipSuccess) {
+        delete m;
+        return hip_fail(e, "hipModuleLoadData");
+    }
+    m->lowered = std::move(prog.lowered);
+    *out = m;
+    return GERN_HIP_OK;
+}
+
+int gern_hip_compile_only(const char *source, const char *const *name_exprs, int n_name_exprs,
+                          const char *const *options, int n_options, const char *arch,
+                          size_t *code_size) {
+    if (arch == nullptr || arch[0] == '\0') {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_compile_only needs an explicit arch");
+    }
+    CompiledProgram prog;
+    int rc = compile_program(source, name_exprs, n_name_exprs, options, n_options, arch, prog);
+    if (rc != GERN_HIP_OK) {
+        return rc;
+    }
+    if (code_size) {
+        *code_size = prog.code.size();
+    }
+    return GERN_HIP_OK;
+}
+
+int gern_hip_get_kernel(gern_hip_module module, const char *name_expr, gern_hip_kernel *out) {
+    if (module == nullptr || name_expr == nullptr || out == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_get_kernel: null argument");
+    }
+    *out = nullptr;
+    auto it = module->lowered.find(name_expr);
+    // A plain (non-template) extern "C" kernel can be looked up directly.
+    std::string symbol = (it != module->lowered.end()) ? it->second : std::string(name_expr);
+    hipFunction_t fn = nullptr;
+    hipError_t e = hipModuleGetFunction(&fn, module->module, symbol.c_str());
+    if (e != hipSuccess) {
+        return hip_fail(e, ("hipModuleGetFunction(" + symbol + ")").c_str());
+    }
+    auto *k = new gern_hip_kernel_s();
+    k->fn = fn;
+    k->name = name_expr;
+    module->kernels.push_back(k);
+    *out = k;
+    return GERN_HIP_OK;
+}
+
+int gern_hip_kernel_info(gern_hip_kernel kernel, int32_t *vgprs, int32_t *sgprs,
+                         int32_t *static_lds_bytes, int32_t *scratch_bytes) {
+    if (kernel == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_kernel_info: null kernel");
+    }
+    int v = 0;
+    if (vgprs) {
+        HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_NUM_REGS, kernel->fn));
+        *vgprs = v;
+    }
+    if (sgprs) {
+        *sgprs = 0;
+    }
+    if (static_lds_bytes) {
+        HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, kernel->fn));
+        *static_lds_bytes = v;
+    }
+    if (scratch_bytes) {
+        HIP_TRY(hipFuncGetAttribute(&v, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, kernel->fn));
+        *scratch_bytes = v;
+    }
+    return GERN_HIP_OK;
+}
+
+int gern_hip_launch(gern_hip_kernel kernel, const uint32_t grid[3], const uint32_t block[3],
+                    uint32_t lds_bytes, void **params, void *stream) {
+    if (kernel == nullptr || grid == nullptr || block == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: null argument");
+    }
+    int rc = load_limits();
+    if (rc != GERN_HIP_OK) {
+        return rc;
+    }
+    uint64_t threads = 1;
+    for (int i = 0; i < 3; i++) {
+        if (grid[i] == 0 || block[i] == 0) {
+            return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: zero-sized grid or block dimension");
+        }
+        if (block[i] > (uint32_t)g_limits.max_block_dim[i]) {
+            return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: block dimension " + std::to_string(i) +
+                                                   " = " + std::to_string(block[i]) + " exceeds the device limit");
+        }
+        if (grid[i] > (uint32_t)g_limits.max_grid_dim[i]) {
+            return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: grid dimension " + std::to_string(i) +
+                                                   " = " + std::to_string(grid[i]) + " exceeds the device limit");
+        }
+        threads *= block[i];
+    }
+    if (threads > (uint64_t)g_limits.max_threads_per_block) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: " + std::to_string(threads) +
+                                               " threads per block exceeds the device limit of " +
+                                               std::to_string(g_limits.max_threads_per_block));
+    }
+    if ((int64_t)lds_bytes > g_limits.lds_bytes_per_block) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: " + std::to_string(lds_bytes) +
+                                               " bytes of LDS exceeds the per-block limit of " +
+                                               std::to_string(g_limits.lds_bytes_per_block));
+    }
+    HIP_TRY(hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                  lds_bytes, (hipStream_t)stream, params, nullptr));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_sync(void) {
+    HIP_TRY(hipDeviceSynchronize());
+    return GERN_HIP_OK;
+}
+
+int gern_hip_stream_sync(void *stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_check(void) {
+    HIP_TRY(hipPeekAtLastError());
+    return GERN_HIP_OK;
+}
+
+int gern_hip_module_unload(gern_hip_module module) {
+    if (module == nullptr) {
+        return GERN_HIP_OK;
+    }
+    hipError_t e = hipModuleUnload(module->module);
+    for (auto *k : module->kernels) {
+        delete k;
+    }
+    delete module;
+    if (e != hipSuccess) {
+        return hip_fail(e, "hipModuleUnload");
+    }
+    return GERN_HIP_OK;
+}
+
+int gern_hip_malloc(void **ptr, size_t bytes) {
+    if (ptr == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_malloc: null output pointer");
+    }
+    HIP_TRY(hipMalloc(ptr, bytes));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_free(void *ptr) {
+    HIP_TRY(hipFree(ptr));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+    HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_memset(void *dst, int value, size_t bytes) {
+    HIP_TRY(hipMemset(dst, value, bytes));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_event_create(gern_hip_event *out) {
+    if (out == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_event_create: null output handle");
+    }
+    auto *ev = new gern_hip_event_s();
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e != hipSuccess) {
+        delete ev;
+        return hip_fail(e, "hipEventCreate");
+    }
+    *out = ev;
+    return GERN_HIP_OK;
+}
+
+int gern_hip_event_record(gern_hip_event ev, void *stream) {
+    if (ev == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_event_record: null event");
+    }
+    HIP_TRY(hipEventRecord(ev->ev, (hipStream_t)stream));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_event_elapsed_ms(gern_hip_event start, gern_hip_event stop, float *ms) {
+    if (start == nullptr || stop == nullptr || ms == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_event_elapsed_ms: null argument");
+    }
+    HIP_TRY(hipEventSynchronize(stop->ev));
+    HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+    return GERN_HIP_OK;
+}
+
+int gern_hip_event_destroy(gern_hip_event ev) {
+    if (ev == nullptr) {
+        return GERN_HIP_OK;
+    }
+    hipError_t e = hipEventDestroy(ev->ev);
+    delete ev;
+    if (e != hipSuccess) {
+        return hip_fail(e, "hipEventDestroy");
+    }
+    return GERN_HIP_OK;
+}
+
+int gern_hip_device_limits(gern_hip_limits *out) {
+    if (out == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_device_limits: null output");
+    }
+    int rc = load_limits();
+    if (rc != GERN_HIP_OK) {
+        return rc;
+    }
+    *out = g_limits;
+    return GERN_HIP_OK;
+}
+
+int gern_hip_device_count(int *count) {
+    if (count == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_device_count: null output");
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    *count = (e == hipSuccess) ? n : 0;
+    return GERN_HIP_OK;
+}
+
+size_t gern_hip_last_error(char *buf, size_t buf_size) {
+    if (buf != nullptr && buf_size > 0) {
+        size_t n = g_last_error.size() < buf_size - 1 ? g_last_error.size() : buf_size - 1;
+        std::memcpy(buf, g_last_error.data(), n);
+        buf[n] = '\0';
+    }
+    return g_last_error.size();
+}
+
+}  // extern "C"

@@ -1,0 +1,131 @@
+// Row-softmax building blocks on wave-distributed register tiles: row maximum,
+// row sum, x - v[row], exp, x / v[row].
+//
+// They are the wavefront-level twins of the reference's softmax gernels
+// (apps/common/impl/impl.h:7-24 exp_matrix, :26-51 divide_vec, :53-78
+// subtract_vec, :80-133 sum_row, :135-188 max_shuffle).  The reference reduces
+// a row with 32-lane shuffles plus a shared-memory hop between warps; here a
+// whole row lives in one 64-lane wavefront, so the reduction is a lane-local
+// scan followed by a DPP / ds_swizzle butterfly that never leaves the wave.
+#pragma once
+
+#include "gernels/wave_tile.h"
+
+namespace gernels {
+
+struct MaxOp {
+    static __device__ __forceinline__ float identity() {
+        return -__builtin_huge_valf();
+    }
+    static __device__ __forceinline__ float apply(float a, float b) {
+        return __builtin_fmaxf(a, b);
+    }
+};
+
+struct SumOp {
+    static __device__ __forceinline__ float identity() {
+        return 0.f;
+    }
+    static __device__ __forceinline__ float apply(float a, float b) {
+        return a + b;
+    }
+};
+
+template<int kCtrl>
+__device__ __forceinline__ float dpp_move(float x) {
+    return as_float(__builtin_amdgcn_update_dpp(as_int(x), as_int(x), kCtrl, 0xf, 0xf, false));
+}
+
+// All-lanes reduction over one wavefront.  Steps 1-4 stay inside a 16-lane DPP
+// row (quad permutes, then half-mirror and mirror); step 5 swaps the two rows
+// of each 32-lane half through ds_swizzle; step 6 combines the two halves by
+// reading one lane of each into scalars, which also leaves the result uniform.
+template<typename Op>
+__device__ __forceinline__ float wave_all_reduce(float x) {
+    x = Op::apply(x, dpp_move<0xB1>(x));   // quad_perm [1,0,3,2]
+    x = Op::apply(x, dpp_move<0x4E>(x));   // quad_perm [2,3,0,1]
+    x = Op::apply(x, dpp_move<0x141>(x));  // row_half_mirror
+    x = Op::apply(x, dpp_move<0x140>(x));  // row_mirror
+    // bit-mode swizzle: and_mask 0x1f, or_mask 0, xor_mask 0x10 -> lane ^ 16
+    x = Op::apply(x, as_float(__builtin_amdgcn_ds_swizzle(as_int(x), 0x401F)));
+    const float lo = as_float(__builtin_amdgcn_readlane(as_int(x), 0));
+    const float hi = as_float(__builtin_amdgcn_readlane(as_int(x), 32));
+    return Op::apply(lo, hi);
+}
+
+template<typename Op, typename TV, typename TI>
+__device__ __forceinline__ void reduce_rows(TV &out, const TI &in) {
+    static_assert(TV::size == TI::rows, "one scalar per tile row");
+    const int lane = lane_id();
+#pragma unroll
+    for (int64_t r = 0; r < TI::rows; r++) {
+        float acc = Op::identity();
+#pragma unroll
+        for (int64_t k = 0; k < TI::chunks; k++) {
+            const float4 t = in.v[r][k];
+            const int64_t lc = k * kWaveCols + 4 * lane;
+            // columns past the tile's logical width do not take part
+            if (lc + 0 < TI::cols) acc = Op::apply(acc, t.x);
+            if (lc + 1 < TI::cols) acc = Op::apply(acc, t.y);
+            if (lc + 2 < TI::cols) acc = Op::apply(acc, t.z);
+            if (lc + 3 < TI::cols) acc = Op::apply(acc, t.w);
+        }
+        out.val[r] = wave_all_reduce<Op>(acc);
+    }
+}
+
+// `stride` (the number of threads sharing a row in the reference's signature)
+// is accepted for source compatibility and ignored: a row is always one wave.
+template<int64_t stride = 64, typename TV, typename TI>
+__device__ __forceinline__ void max_row(TV &out, const TI &in) {
+    reduce_rows<MaxOp>(out, in);
+}
+
+template<int64_t stride = 64, typename TV, typename TI>
+__device__ __forceinline__ void sum_row(TV &out, const TI &in) {
+    reduce_rows<SumOp>(out, in);
+}
+
+template<typename TV, typename T>
+__device__ __forceinline__ void subtract_vec(const TV &vec, const T &in, T &out) {
+    static_assert(TV::size == T::rows, "one scalar per tile row");
+#pragma unroll
+    for (int64_t r = 0; r < T::rows; r++) {
+        const float s = vec.val[r];
+#pragma unroll
+        for (int64_t k = 0; k < T::chunks; k++) {
+            const float4 t = in.v[r][k];
+            out.v[r][k] = make_float4(t.x - s, t.y - s, t.z - s, t.w - s);
+        }
+    }
+}
+
+template<typename T>
+__device__ __forceinline__ void exp_matrix(const T &in, T &out) {
+#pragma unroll
+    for (int64_t r = 0; r < T::rows; r++) {
+#pragma unroll
+        for (int64_t k = 0; k < T::chunks; k++) {
+            const float4 t = in.v[r][k];
+            out.v[r][k] = make_float4(expf(t.x), expf(t.y), expf(t.z), expf(t.w));
+        }
+    }
+}
+
+template<typename TV, typename T>
+__device__ __forceinline__ void divide_vec(const TV &vec, const T &in, T &out) {
+    static_assert(TV::size == T::rows, "one scalar per tile row");
+#pragma unroll
+    for (int64_t r = 0; r < T::rows; r++) {
+        const float d = vec.val[r];
+        const float rcp = 1.0f / d;  // one IEEE division per row
+#pragma unroll
+        for (int64_t k = 0; k < T::chunks; k++) {
+            const float4 t = in.v[r][k];
+            out.v[r][k] = make_float4(div_by(t.x, d, rcp), div_by(t.y, d, rcp), div_by(t.z, d, rcp),
+                                      div_by(t.w, d, rcp));
+        }
+    }
+}
+
+}  // namespace gernels

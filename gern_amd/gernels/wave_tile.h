@@ -1,0 +1,135 @@
+// Wave-distributed register tiles and the global fp32 matrix they are cut from.
+//
+// A WaveTile<R, C> is an R x C fp32 tile owned by ONE 64-lane wavefront and
+// held entirely in VGPRs: lane l keeps, for every row and every 256-column
+// chunk k, the float4 covering columns 256*k + 4*l .. 256*k + 4*l + 3.  One
+// row of a chunk is therefore one fully coalesced 1 KiB access (64 lanes x
+// 16 B), which is how MatrixF32 loads and stores it.
+//
+// This is the gfx950 counterpart of the per-thread StaticMatrix register tile
+// of the reference (apps/common/impl/gpu-matrix-const.h:29-38, query :131-150,
+// insert :152-170, allocate_static :251-254): the same query / allocate /
+// insert contract that generated code calls, re-laid-out so that the unit that
+// owns a tile is a wavefront rather than a thread and neighbouring columns
+// live in neighbouring lanes (one DPP move away) rather than in a halo that
+// every thread re-reads from memory.
+#pragma once
+
+#include "gernels/prelude.h"
+
+namespace gernels {
+
+template<int64_t R, int64_t C>
+struct WaveTile {
+    static constexpr int64_t rows = R;
+    static constexpr int64_t cols = C;
+    static constexpr int64_t chunks = (C + kWaveCols - 1) / kWaveCols;
+    float4 v[R][chunks];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+// Per-row scalars (row maxima, row sums), replicated in every lane.
+template<int64_t R>
+struct WaveVec {
+    static constexpr int64_t size = R;
+    float val[R];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+template<int64_t R, int64_t C>
+__device__ __forceinline__ WaveTile<R, C> allocate_wave_tile() {
+    return WaveTile<R, C>();
+}
+
+template<int64_t R>
+__device__ __forceinline__ WaveVec<R> allocate_wave_vec() {
+    return WaveVec<R>();
+}
+
+// Row-major fp32 matrix in HBM.  Plain aggregate: the host fills one in and
+// the launch passes it by value, so host and device layouts must agree
+// (pointer, then three 64-bit integers).
+struct MatrixF32 {
+    float *data;
+    int64_t row;
+    int64_t col;
+    int64_t lda;
+
+    // Loads the R x C tile whose top-left element is (x, y).  Elements outside
+    // the matrix read as 0; a tile may therefore hang over the right or bottom
+    // edge (ragged last tile of a grid).
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ WaveTile<R, C> load_wave(int64_t x, int64_t y) const {
+        WaveTile<R, C> t;
+        const int lane = lane_id();
+#pragma unroll
+        for (int64_t r = 0; r < R; r++) {
+            const int64_t rr = x + r;
+            const bool row_ok = rr < row;
+            const float *p = data + rr * lda + y;
+            // A row can use 16-byte accesses when its first element is 16-byte
+            // aligned; the test is wave-uniform.
+            const bool vec_ok = (((uint64_t)p) & 15u) == 0;
+#pragma unroll
+            for (int64_t k = 0; k < WaveTile<R, C>::chunks; k++) {
+                const int64_t lc = k * kWaveCols + 4 * lane;  // column inside the tile
+                const int64_t cc = y + lc;                    // column inside the matrix
+                float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (row_ok && lc < C) {
+                    if (vec_ok && cc + 3 < col) {
+                        val = *reinterpret_cast<const float4 *>(p + lc);
+                    } else {
+                        if (cc + 0 < col) val.x = p[lc + 0];
+                        if (cc + 1 < col) val.y = p[lc + 1];
+                        if (cc + 2 < col) val.z = p[lc + 2];
+                        if (cc + 3 < col) val.w = p[lc + 3];
+                    }
+                }
+                t.v[r][k] = val;
+            }
+        }
+        return t;
+    }
+
+    // An output tile: nothing is read, the producer overwrites every element.
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ WaveTile<R, C> view_wave(int64_t, int64_t) const {
+        return WaveTile<R, C>();
+    }
+
+    // Stores the tile at (x, y), clipped to the tile's logical width C and to
+    // the matrix bounds.
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ void store_wave(int64_t x, int64_t y, const WaveTile<R, C> &t) const {
+        const int lane = lane_id();
+#pragma unroll
+        for (int64_t r = 0; r < R; r++) {
+            const int64_t rr = x + r;
+            if (rr >= row) {
+                continue;
+            }
+            float *p = data + rr * lda + y;
+            const bool vec_ok = (((uint64_t)p) & 15u) == 0;
+#pragma unroll
+            for (int64_t k = 0; k < WaveTile<R, C>::chunks; k++) {
+                const int64_t lc = k * kWaveCols + 4 * lane;
+                const int64_t cc = y + lc;
+                const float4 val = t.v[r][k];
+                if (vec_ok && lc + 3 < C && cc + 3 < col) {
+                    *reinterpret_cast<float4 *>(p + lc) = val;
+                } else {
+                    if (lc + 0 < C && cc + 0 < col) p[lc + 0] = val.x;
+                    if (lc + 1 < C && cc + 1 < col) p[lc + 1] = val.y;
+                    if (lc + 2 < C && cc + 2 < col) p[lc + 2] = val.z;
+                    if (lc + 3 < C && cc + 3 < col) p[lc + 3] = val.w;
+                }
+            }
+        }
+    }
+};
+
+}  // namespace gernels

@@ -1,0 +1,3 @@
+// Forwarding header: keeps the reference's include path working.
+#pragma once
+#include "gern/core/abstract_function.h"
