@@ -1,0 +1,245 @@
+"""gern_amd: Gern's fused kernels on MI355X (gfx950).
+
+This Python module is a thin ctypes view of the package's C ABI
+(include/gern_hip.h, include/gern_pipelines.h) for tests, the smoke check and
+the benchmark.  The product is the native code: Gern's C++ front end, the HIP
+code generator and Runner (libgern.so), the hiprtc/hipModule runtime behind a C
+ABI (libgern_hip.so), the hand-written gernels (gernels/*.h) and the composed
+pipelines (libgern_pipelines.so).
+
+There is no CPU fallback: every compute entry point raises if the native
+libraries or a GPU are missing.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+COMPILE_ONLY = 1
+NO_XCD_REMAP = 2
+
+_libs = None
+
+
+class GernError(RuntimeError):
+    pass
+
+
+def _load():
+    """Loads the native libraries (built in-tree by gern_amd/build.py)."""
+    global _libs
+    if _libs is not None:
+        return _libs
+    # PyTorch ships its own HIP runtime under the same sonames.  Loading it
+    # first makes the whole process share ONE runtime; two runtimes in one
+    # process each open the device and the second one finds no GPU.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    paths = {n: os.path.join(_HERE, "lib%s.so" % n) for n in ("gern_hip", "gern", "gern_pipelines")}
+    for n, p in paths.items():
+        if not os.path.exists(p):
+            raise GernError("%s is missing: run `python gern_amd/build.py` (or __graft_entry__.build())" % p)
+    hip = C.CDLL(paths["gern_hip"], mode=C.RTLD_GLOBAL)
+    C.CDLL(paths["gern"], mode=C.RTLD_GLOBAL)
+    pipes = C.CDLL(paths["gern_pipelines"], mode=C.RTLD_GLOBAL)
+
+    i64, vp, sz = C.c_int64, C.c_void_p, C.c_size_t
+    hip.gern_hip_last_error.restype = sz
+    hip.gern_hip_last_error.argtypes = [C.c_char_p, sz]
+    pipes.gern_pipelines_last_error.restype = sz
+    pipes.gern_pipelines_last_error.argtypes = [C.c_char_p, sz]
+    pipes.gern_pipeline_source.restype = C.c_char_p
+    pipes.gern_pipeline_source.argtypes = [vp]
+    pipes.gern_pipeline_kernel_name.restype = C.c_char_p
+    pipes.gern_pipeline_kernel_name.argtypes = [vp]
+    pipes.gern_pipeline_destroy.argtypes = [vp]
+    pipes.gern_blur_chain_create.argtypes = [C.c_char_p, i64, i64, i64, C.c_int, C.c_int, C.POINTER(vp)]
+    pipes.gern_blur_chain_run.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
+    pipes.gern_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
+    pipes.gern_softmax_run.argtypes = [vp, vp, vp, i64, i64, vp]
+    if hasattr(pipes, "gern_gemm_create"):
+        pipes.gern_gemm_create.argtypes = [C.c_int, C.c_int, C.POINTER(vp)]
+        pipes.gern_gemm_run.argtypes = [vp, vp, vp, vp, i64, i64, i64, vp]
+    if hasattr(pipes, "gern_qk_softmax_create"):
+        pipes.gern_qk_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
+        pipes.gern_qk_softmax_run.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
+    hip.gern_hip_event_create.argtypes = [C.POINTER(vp)]
+    hip.gern_hip_event_record.argtypes = [vp, vp]
+    hip.gern_hip_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]
+    hip.gern_hip_event_destroy.argtypes = [vp]
+    hip.gern_hip_stream_sync.argtypes = [vp]
+    _libs = (hip, pipes)
+    return _libs
+
+
+def hip_lib():
+    return _load()[0]
+
+
+def pipelines_lib():
+    return _load()[1]
+
+
+def _pipe_error():
+    n = pipelines_lib().gern_pipelines_last_error(None, 0)
+    buf = C.create_string_buffer(n + 1)
+    pipelines_lib().gern_pipelines_last_error(buf, n + 1)
+    return buf.value.decode(errors="replace")
+
+
+def _hip_error():
+    n = hip_lib().gern_hip_last_error(None, 0)
+    buf = C.create_string_buffer(n + 1)
+    hip_lib().gern_hip_last_error(buf, n + 1)
+    return buf.value.decode(errors="replace")
+
+
+def _check(rc):
+    if rc != 0:
+        raise GernError(_pipe_error())
+
+
+class Limits(C.Structure):
+    _fields_ = [("wavefront_size", C.c_int32), ("max_threads_per_block", C.c_int32),
+                ("max_block_dim", C.c_int32 * 3), ("max_grid_dim", C.c_int32 * 3),
+                ("lds_bytes_per_block", C.c_int64), ("compute_units", C.c_int32), ("clock_khz", C.c_int32),
+                ("hbm_bytes", C.c_int64), ("arch", C.c_char * 64)]
+
+
+def device_limits():
+    lim = Limits()
+    if hip_lib().gern_hip_device_limits(C.byref(lim)) != 0:
+        raise GernError(_hip_error())
+    return lim
+
+
+def device_count():
+    n = C.c_int(0)
+    hip_lib().gern_hip_device_count(C.byref(n))
+    return n.value
+
+
+class Event:
+    """A HIP event recorded on the stream the kernels are launched on."""
+
+    def __init__(self):
+        self.h = C.c_void_p()
+        if hip_lib().gern_hip_event_create(C.byref(self.h)) != 0:
+            raise GernError(_hip_error())
+
+    def record(self, stream=None):
+        if hip_lib().gern_hip_event_record(self.h, stream) != 0:
+            raise GernError(_hip_error())
+
+    def elapsed_ms_until(self, stop):
+        ms = C.c_float()
+        if hip_lib().gern_hip_event_elapsed_ms(self.h, stop.h, C.byref(ms)) != 0:
+            raise GernError(_hip_error())
+        return ms.value
+
+    def __del__(self):
+        try:
+            hip_lib().gern_hip_event_destroy(self.h)
+        except Exception:
+            pass
+
+
+def _ptr(t):
+    """Device pointer of a torch tensor (or a raw integer address)."""
+    return C.c_void_p(t if isinstance(t, int) else t.data_ptr())
+
+
+class _Pipeline:
+    def __init__(self):
+        self.h = C.c_void_p()
+
+    @property
+    def source(self):
+        return pipelines_lib().gern_pipeline_source(self.h).decode()
+
+    @property
+    def kernel_name(self):
+        return pipelines_lib().gern_pipeline_kernel_name(self.h).decode()
+
+    def __del__(self):
+        try:
+            if self.h:
+                pipelines_lib().gern_pipeline_destroy(self.h)
+        except Exception:
+            pass
+
+
+class BlurChain(_Pipeline):
+    """Fused separable box blur, e.g. BlurChain("xyx")."""
+
+    def __init__(self, pattern, stride=3, tile_rows=8, tile_cols=None, waves_per_block=1, flags=0):
+        super().__init__()
+        nx = pattern.count("x")
+        if tile_cols is None:
+            tile_cols = (256 - nx * (stride - 1)) // 4 * 4
+        self.pattern, self.stride = pattern, stride
+        self.nx, self.ny = nx, pattern.count("y")
+        _check(pipelines_lib().gern_blur_chain_create(pattern.encode(), stride, tile_rows, tile_cols,
+                                                      waves_per_block, flags, C.byref(self.h)))
+
+    def out_shape(self, rows, cols):
+        return rows - self.ny * (self.stride - 1), cols - self.nx * (self.stride - 1)
+
+    def __call__(self, img, out, stream=None):
+        """img, out: contiguous fp32 CUDA tensors; out has out_shape(*img.shape)."""
+        rows, cols = img.shape
+        assert tuple(out.shape) == self.out_shape(rows, cols)
+        _check(pipelines_lib().gern_blur_chain_run(self.h, _ptr(img), rows, cols, img.stride(0), _ptr(out),
+                                                   out.stride(0), stream))
+        return out
+
+
+class Softmax(_Pipeline):
+    """Fused row softmax over matrices with `ncol` columns."""
+
+    def __init__(self, ncol, rows_per_wave=1, flags=0):
+        super().__init__()
+        self.ncol = ncol
+        _check(pipelines_lib().gern_softmax_create(ncol, rows_per_wave, flags, C.byref(self.h)))
+
+    def __call__(self, x, out, stream=None):
+        rows, cols = x.shape
+        assert cols == self.ncol and tuple(out.shape) == (rows, cols) and x.stride(0) == out.stride(0)
+        _check(pipelines_lib().gern_softmax_run(self.h, _ptr(x), _ptr(out), rows, x.stride(0), stream))
+        return out
+
+
+class Gemm(_Pipeline):
+    """C += A @ B.  variant "f32" (vector ALU) or "bf16" (MFMA, fp32 accumulate)."""
+
+    def __init__(self, variant="f32", flags=0):
+        super().__init__()
+        self.variant = variant
+        _check(pipelines_lib().gern_gemm_create({"f32": 0, "bf16": 1}[variant], flags, C.byref(self.h)))
+
+    def __call__(self, A, B, Cm, stream=None):
+        M, K = A.shape
+        N = B.shape[1]
+        assert tuple(B.shape) == (K, N) and tuple(Cm.shape) == (M, N)
+        assert A.is_contiguous() and B.is_contiguous() and Cm.is_contiguous()
+        _check(pipelines_lib().gern_gemm_run(self.h, _ptr(A), _ptr(B), _ptr(Cm), M, N, K, stream))
+        return Cm
+
+
+class QKSoftmax(_Pipeline):
+    """S = softmax_rows(scale * Q @ K^T), Q and K in bf16, S in fp32."""
+
+    def __init__(self, head_dim=128, max_keys=4096, flags=0):
+        super().__init__()
+        self.head_dim = head_dim
+        _check(pipelines_lib().gern_qk_softmax_create(head_dim, max_keys, flags, C.byref(self.h)))
+
+    def __call__(self, Q, K, S, scale, stream=None):
+        M, D = Q.shape
+        N = K.shape[0]
+        assert D == self.head_dim and K.shape[1] == D and tuple(S.shape) == (M, N)
+        assert Q.is_contiguous() and K.is_contiguous() and S.is_contiguous()
+        _check(pipelines_lib().gern_qk_softmax_run(self.h, _ptr(Q), _ptr(K), _ptr(S), M, N, float(scale), stream))
+        return S

@@ -1,0 +1,149 @@
+// Annotations of the block GEMM gernels (gernels/mm.h).
+//
+// The dependency pattern is the reference's (test/library/matrix/annot/cpu-matrix.h:258-303,
+// gernels/mm/gern_annot/functions.h:7-100): to produce C[i..i+ti, j..j+tj] the
+// function consumes, for every k step of a reducible loop over k_dim,
+// A[i..i+ti, k..k+tk] and B[k..k+tk, j..j+tj].
+#pragma once
+
+#include "annot/matrix.h"
+
+namespace gern {
+namespace annot {
+
+// A GEMM operand in HBM; its subsets are windows (no data movement).
+class MatrixOperand : public AbstractDataType {
+public:
+    enum Element { F32, BF16 };
+    MatrixOperand(const std::string &name, Element element)
+        : name(name), element(element) {
+    }
+    std::string getName() const override {
+        return name;
+    }
+    std::string getType() const override {
+        return element == BF16 ? "gernels::MatrixBF16" : "gernels::MatrixF32";
+    }
+    std::vector<Variable> getFields() const override {
+        return {x, y, row, col};
+    }
+    FunctionSignature getAllocateFunction() const override {
+        return FunctionSignature{.name = "unsupported_allocate"};
+    }
+    FunctionSignature getFreeFunction() const override {
+        return FunctionSignature{.name = "destroy"};
+    }
+    FunctionSignature getInsertFunction() const override {
+        return FunctionSignature{.name = "unsupported_insert"};
+    }
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{
+            .name = "template view",
+            .args = {x, y},
+            .template_args = {row, col},
+        };
+    }
+    bool readMember(const void *object, const std::string &member, int64_t &value) const override {
+        // MatrixF32 and MatrixBF16 share their layout
+        return MatrixF32("", MatrixF32::INPUT).readMember(object, member, value);
+    }
+
+private:
+    std::string name;
+    Element element;
+    Variable x{"x"};
+    Variable y{"y"};
+    Variable row{"row", Datatype::Int64, true};
+    Variable col{"col", Datatype::Int64, true};
+};
+
+// The GEMM result in HBM; its subsets are block-distributed accumulator tiles
+// (loaded from C, so the product is added to what C holds, and stored back).
+class MatrixAccumulator : public AbstractDataType {
+public:
+    enum Engine { FMA, MFMA };
+    MatrixAccumulator(const std::string &name, Engine engine)
+        : name(name), engine(engine) {
+    }
+    std::string getName() const override {
+        return name;
+    }
+    std::string getType() const override {
+        return "gernels::MatrixF32";
+    }
+    std::vector<Variable> getFields() const override {
+        return {x, y, row, col};
+    }
+    FunctionSignature getAllocateFunction() const override {
+        return FunctionSignature{.name = "unsupported_allocate"};
+    }
+    FunctionSignature getFreeFunction() const override {
+        return FunctionSignature{.name = "destroy"};
+    }
+    FunctionSignature getInsertFunction() const override {
+        return FunctionSignature{
+            .name = "store_acc",
+            .args = {x, y},
+        };
+    }
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{
+            .name = engine == MFMA ? "template load_acc_mfma" : "template load_acc_fma",
+            .args = {x, y},
+            .template_args = {row, col},
+        };
+    }
+    bool insertQuery() const override {
+        return true;
+    }
+    bool readMember(const void *object, const std::string &member, int64_t &value) const override {
+        return MatrixF32("", MatrixF32::INPUT).readMember(object, member, value);
+    }
+
+private:
+    std::string name;
+    Engine engine;
+    Variable x{"x"};
+    Variable y{"y"};
+    Variable row{"row", Datatype::Int64, true};
+    Variable col{"col", Datatype::Int64, true};
+};
+
+// C += A * B on one workgroup.  Bind "k_dim" to the variable that holds the
+// reduction extent, and Reduce over it.
+class MatrixMultiply : public AbstractFunction {
+public:
+    MatrixMultiply(AbstractDataTypePtr A, AbstractDataTypePtr B, AbstractDataTypePtr C)
+        : A(A), B(B), C(C) {
+    }
+    Annotation getAnnotation() override {
+        Variable i("i"), j("j"), k("k");
+        Variable ti("ti", Datatype::Int64, true), tj("tj", Datatype::Int64, true), tk("tk", Datatype::Int64, true);
+        return Tileable(i = Expr(0), ADTMember(C, "row", false), ti,
+                        Tileable(j = Expr(0), ADTMember(C, "col", false), tj,
+                                 Produces::Subset(C, {i, j, ti, tj}),
+                                 Consumes::Subsets(Reducible(k = Expr(0), k_dim, tk,
+                                                             SubsetObjMany({
+                                                                 SubsetObj(A, {i, k, ti, tk}),
+                                                                 SubsetObj(B, {k, j, tk, tj}),
+                                                             })))))
+            // all threads of a workgroup cooperate
+            .occupies({Grid::Unit::THREAD_X});
+    }
+    FunctionSignature getFunction() override {
+        FunctionSignature f;
+        f.name = "gernels::matrix_multiply";
+        f.args = {Parameter(A), Parameter(B), Parameter(C)};
+        return f;
+    }
+    std::vector<std::string> getHeader() override {
+        return {"gernels/mm.h"};
+    }
+
+private:
+    AbstractDataTypePtr A, B, C;
+    Variable k_dim{"k_dim", Datatype::Int64};
+};
+
+}  // namespace annot
+}  // namespace gern

@@ -1,0 +1,58 @@
+"""Builds the native libraries of the package, in-tree.
+
+    libgern_hip.so        C ABI over hiprtc / hipModule (include/gern_hip.h)
+    libgern.so            Gern's C++ front end, code generator and Runner
+    libgern_pipelines.so  C ABI over the fused pipelines (include/gern_pipelines.h)
+
+and ahead-of-time compiles every gernel header for gfx950 as a build check
+(the kernels that actually run are instantiated by hiprtc from generated code).
+"""
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+CXXFLAGS = ["-std=c++20", "-O2", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
+            "-I" + os.path.join(HERE, "include"), "-I" + os.path.join(HERE, "include", "gern"),
+            "-I" + HERE, "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROCM, "include")]
+# Packed-FP32 instructions are kept out of every kernel.
+HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+            "-packed-fp32-ops", "-I" + HERE]
+
+
+def run(cmd):
+    print("+ " + " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_native():
+    rpath = "-Wl,-rpath,$ORIGIN:" + os.path.join(ROCM, "lib")
+    run(["g++"] + CXXFLAGS + ["-shared", os.path.join(HERE, "csrc", "gern_hip.cpp"),
+                               "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lhiprtc", rpath,
+                               "-o", os.path.join(HERE, "libgern_hip.so")])
+    srcs = sorted(glob.glob(os.path.join(HERE, "src", "*.cpp")))
+    run(["g++"] + CXXFLAGS + ["-shared"] + srcs + ["-L" + HERE, "-lgern_hip", "-ldl", rpath,
+                                                  "-o", os.path.join(HERE, "libgern.so")])
+    run(["g++"] + CXXFLAGS + ["-shared", os.path.join(HERE, "csrc", "pipelines.cpp"), "-L" + HERE, "-lgern",
+                               "-lgern_hip", "-ldl", rpath, "-o", os.path.join(HERE, "libgern_pipelines.so")])
+
+
+def build_gernel_check():
+    """hipcc cross-compiles an instantiation of every gernel for gfx950."""
+    src = os.path.join(HERE, "csrc", "gernel_check.hip")
+    out = os.path.join(HERE, "csrc", "gernel_check.o")
+    run([os.path.join(ROCM, "bin", "hipcc")] + HIPFLAGS + ["-c", "--cuda-device-only", src, "-o", out])
+
+
+def build_all():
+    build_native()
+    build_gernel_check()
+
+
+if __name__ == "__main__":
+    build_all()
+    print("build ok")

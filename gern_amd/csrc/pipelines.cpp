@@ -1,0 +1,434 @@
+// C ABI over the fused pipelines (include/gern_pipelines.h).  Everything here
+// is written against Gern's C++ API, the way a user application is: declare
+// data structures, compose annotated functions, compile with a Runner,
+// evaluate with the caller's buffers.
+#include "gern_pipelines.h"
+
+#include "annot/blur.h"
+#include "annot/mm.h"
+#include "annot/qk_softmax.h"
+#include "annot/softmax.h"
+#include "gern/codegen/codegen.h"
+#include "gern_hip.h"
+
+#include <dlfcn.h>
+
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <string>
+
+using namespace gern;
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(const std::string &msg) {
+    g_error = msg;
+    return 1;
+}
+
+// Directory that holds this library; the gernel headers live next to it.
+std::string packageDir() {
+    Dl_info info;
+    if (dladdr((const void *)&packageDir, &info) && info.dli_fname) {
+        std::string path(info.dli_fname);
+        auto slash = path.rfind('/');
+        return slash == std::string::npos ? "." : path.substr(0, slash);
+    }
+    return ".";
+}
+
+AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
+    return AbstractDataTypePtr(new const annot::MatrixF32(name, role));
+}
+
+}  // namespace
+
+struct gern_pipeline_s {
+    enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
+    std::unique_ptr<Runner> runner;  // null in compile-only mode
+    std::string source;
+    std::string kernel_name;
+    // blur
+    int64_t nx = 0, ny = 0, stride = 0;
+    // softmax / qk
+    int64_t ncol = 0;
+    int64_t head_dim = 0;
+    // parameter names
+    std::vector<std::string> names;
+};
+
+namespace {
+
+// Generates (and, unless compile-only, loads) the program.
+int finish(gern_pipeline_s *p, Composable program, int flags) {
+    const std::string include = "-I " + packageDir();
+    try {
+        if (flags & GERN_PIPELINE_COMPILE_ONLY) {
+            codegen::GeneratorOptions go;
+            go.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+            codegen::CodeGenerator cg(std::nullopt, go);
+            p->source = cg.generate_code(program);
+            p->kernel_name = cg.getLaunchPlan().name_expression;
+            p->names = cg.getArgumentOrder();
+            const std::string inc = "-I" + packageDir();
+            const char *names[1] = {p->kernel_name.c_str()};
+            const char *opts[1] = {inc.c_str()};
+            size_t size = 0;
+            if (gern_hip_compile_only(p->source.c_str(), names, 1, opts, 1, "gfx950", &size) != 0) {
+                std::string msg(gern_hip_last_error(nullptr, 0) + 1, '\0');
+                gern_hip_last_error(msg.data(), msg.size());
+                return fail("Compilation Failed\n" + msg);
+            }
+            return 0;
+        }
+        p->runner = std::make_unique<Runner>(program);
+        Runner::Options options;
+        options.filename = "";  // keep the source in memory only
+        options.include = include;
+        options.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+        p->runner->compile(options);
+        p->source = p->runner->getSource();
+        p->names = p->runner->getArgumentOrder();
+        return 0;
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_rows, int64_t tile_cols,
+                           int waves_per_block, int flags, gern_pipeline *out) {
+    if (out == nullptr || pattern == nullptr) {
+        return fail("gern_blur_chain_create: null argument");
+    }
+    *out = nullptr;
+    const std::string pat(pattern);
+    int64_t nx = 0, ny = 0;
+    for (char ch : pat) {
+        if (ch == 'x') {
+            nx++;
+        } else if (ch == 'y') {
+            ny++;
+        } else {
+            return fail("gern_blur_chain_create: pattern must consist of 'x' and 'y'");
+        }
+    }
+    if (pat.empty() || stride < 1 || stride > 5 || tile_rows < 1 || tile_cols < 1 || waves_per_block < 1 ||
+        waves_per_block > 16) {
+        return fail("gern_blur_chain_create: bad stride, tile or workgroup shape");
+    }
+    if (tile_cols % 4 != 0 || tile_cols + nx * (stride - 1) > 256) {
+        return fail("gern_blur_chain_create: tile_cols must be a multiple of 4 and tile_cols + halo <= 256");
+    }
+    auto p = std::make_unique<gern_pipeline_s>();
+    p->kind = gern_pipeline_s::BLUR;
+    p->nx = nx;
+    p->ny = ny;
+    p->stride = stride;
+    try {
+        auto input = f32("input", annot::MatrixF32::INPUT);
+        auto output = f32("output", annot::MatrixF32::OUTPUT);
+        Variable stride_v("stride"), row("row"), col("col"), col_block("col_block"), wave("wave");
+        std::vector<Composable> stages;
+        AbstractDataTypePtr prev = input;
+        for (size_t s = 0; s < pat.size(); s++) {
+            AbstractDataTypePtr next =
+                (s + 1 == pat.size()) ? output : f32("stage" + std::to_string(s), annot::MatrixF32::TEMP);
+            std::map<std::string, Variable> bind{{"stride", stride_v.bind(stride)}};
+            if (pat[s] == 'x') {
+                annot::BlurX f{prev, next};
+                stages.push_back(f[bind](prev, next));
+            } else {
+                annot::BlurY f{prev, next};
+                stages.push_back(f[bind](prev, next));
+            }
+            prev = next;
+        }
+        Composable chain(new const Computation(stages));
+        Composable program;
+        if (waves_per_block == 1) {
+            program = Global((Tile(output["row"], row.bind(tile_rows)) || Grid::BLOCK_Y)(
+                                 (Tile(output["col"], col.bind(tile_cols)) || Grid::BLOCK_X)(chain)),
+                             {{Grid::BLOCK_DIM_X, wave.bind(Grid::kWavefrontSize)}});
+        } else {
+            program = Global((Tile(output["row"], row.bind(tile_rows)) || Grid::BLOCK_Y)(
+                (Tile(output["col"], col_block.bind(tile_cols * waves_per_block)) || Grid::BLOCK_X)(
+                    (Tile(output["col"], col.bind(tile_cols)) || Grid::WARP_X)(chain))));
+        }
+        int rc = finish(p.get(), program, flags);
+        if (rc != 0) {
+            return rc;
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    *out = p.release();
+    return 0;
+}
+
+int gern_blur_chain_run(gern_pipeline p, const float *in, int64_t rows, int64_t cols, int64_t ld_in,
+                        float *out, int64_t ld_out, void *stream) {
+    if (p == nullptr || p->kind != gern_pipeline_s::BLUR || in == nullptr || out == nullptr) {
+        return fail("gern_blur_chain_run: bad pipeline or null buffer");
+    }
+    if (!p->runner) {
+        return fail("gern_blur_chain_run: the pipeline was created compile-only");
+    }
+    const int64_t out_rows = rows - p->ny * (p->stride - 1);
+    const int64_t out_cols = cols - p->nx * (p->stride - 1);
+    if (out_rows <= 0 || out_cols <= 0 || ld_in < cols || ld_out < out_cols) {
+        return fail("gern_blur_chain_run: the image is smaller than the stencil footprint, or a bad row stride");
+    }
+    hip::MatrixF32 input{const_cast<float *>(in), rows, cols, ld_in};
+    hip::MatrixF32 output{out, out_rows, out_cols, ld_out};
+    try {
+        p->runner->setStream(stream);
+        p->runner->evaluate({{"input", &input}, {"output", &output}});
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    return 0;
+}
+
+int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pipeline *out) {
+    if (out == nullptr) {
+        return fail("gern_softmax_create: null argument");
+    }
+    *out = nullptr;
+    if (ncol < 1 || ncol > 8192 || rows_per_wave < 1 || rows_per_wave * ((ncol + 255) / 256) > 32) {
+        return fail("gern_softmax_create: a wavefront holds at most 32 x 256 columns of rows in registers");
+    }
+    auto p = std::make_unique<gern_pipeline_s>();
+    p->kind = gern_pipeline_s::SOFTMAX;
+    p->ncol = ncol;
+    try {
+        using M = annot::MatrixF32;
+        auto input = f32("input", M::INPUT);
+        auto output = f32("output", M::OUTPUT);
+        auto shifted = f32("shifted", M::TEMP);
+        auto expd = f32("expd", M::TEMP);
+        auto row_max = AbstractDataTypePtr(new const annot::WaveVec("row_max"));
+        auto row_sum = AbstractDataTypePtr(new const annot::WaveVec("row_sum"));
+        Variable rows("rows"), ncol_v("ncol"), wave("wave");
+        annot::MaxRow max_row{input, row_max};
+        annot::SubtractVec sub{row_max, input, shifted};
+        annot::ExpMatrix ex{shifted, expd};
+        annot::SumRow sum_row{expd, row_sum};
+        annot::DivideVec div{row_sum, expd, output};
+        std::map<std::string, Variable> width{{"ncol", ncol_v.bind(ncol)}};
+        Composable program =
+            Global((Tile(output["row"], rows.bind(rows_per_wave)) || Grid::BLOCK_X)(
+                       Tile(output["col"], ncol_v.bind(ncol))(max_row[width](row_max, input), sub(row_max, input, shifted),
+                                                              ex(shifted, expd), sum_row[width](row_sum, expd),
+                                                              div(row_sum, expd, output))),
+                   {{Grid::BLOCK_DIM_X, wave.bind(Grid::kWavefrontSize)}});
+        // Rows are contiguous and independent: plain launch order already
+        // streams through memory, and measures faster than the XCD order.
+        int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
+        if (rc != 0) {
+            return rc;
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    *out = p.release();
+    return 0;
+}
+
+int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows, int64_t ld, void *stream) {
+    if (p == nullptr || p->kind != gern_pipeline_s::SOFTMAX || in == nullptr || out == nullptr) {
+        return fail("gern_softmax_run: bad pipeline or null buffer");
+    }
+    if (!p->runner) {
+        return fail("gern_softmax_run: the pipeline was created compile-only");
+    }
+    if (rows < 1 || ld < p->ncol) {
+        return fail("gern_softmax_run: bad shape");
+    }
+    hip::MatrixF32 input{const_cast<float *>(in), rows, p->ncol, ld};
+    hip::MatrixF32 output{out, rows, p->ncol, ld};
+    try {
+        p->runner->setStream(stream);
+        p->runner->evaluate({{"input", &input}, {"output", &output}});
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    return 0;
+}
+
+int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
+    if (out == nullptr) {
+        return fail("gern_gemm_create: null argument");
+    }
+    *out = nullptr;
+    if (variant != 0 && variant != 1) {
+        return fail("gern_gemm_create: variant must be 0 (fp32, vector ALU) or 1 (bf16 in, fp32 accumulate, MFMA)");
+    }
+    auto p = std::make_unique<gern_pipeline_s>();
+    p->kind = variant == 1 ? gern_pipeline_s::GEMM_BF16 : gern_pipeline_s::GEMM_F32;
+    try {
+        const bool mfma = variant == 1;
+        // Workgroup tile and the LDS its two pipeline stages need
+        // (gernels/mm.h: mfma_lds_bytes / fma_lds_bytes).
+        const int64_t bm = mfma ? 128 : 128, bn = mfma ? 128 : 128;
+        const int64_t lds = mfma ? 2 * (bm + bn) * 144 : 2 * 2 * 16 * 132 * 4;
+        auto A = AbstractDataTypePtr(new const annot::MatrixOperand(
+            "A", mfma ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32));
+        auto B = AbstractDataTypePtr(new const annot::MatrixOperand(
+            "B", mfma ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32));
+        auto C = AbstractDataTypePtr(new const annot::MatrixAccumulator(
+            "C", mfma ? annot::MatrixAccumulator::MFMA : annot::MatrixAccumulator::FMA));
+        Variable ti("ti"), tj("tj"), tk("tk"), k_dim("k_dim"), threads("threads"), smem("smem");
+        annot::MatrixMultiply mm{A, B, C};
+        // One call walks a whole 4096-deep K chunk, pipelined inside the gernel.
+        Composable program = Global(
+            (Tile(C["row"], ti.bind(bm)) || Grid::BLOCK_Y)((Tile(C["col"], tj.bind(bn)) || Grid::BLOCK_X)(
+                Reduce(k_dim, tk.bind(4096))(mm[{{"k_dim", k_dim}}](A, B, C)))),
+            {{Grid::BLOCK_DIM_X, threads.bind(256)}}, smem.bind(lds));
+        int rc = finish(p.get(), program, flags);
+        if (rc != 0) {
+            return rc;
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    *out = p.release();
+    return 0;
+}
+
+int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64_t M, int64_t N, int64_t K,
+                  void *stream) {
+    if (p == nullptr || (p->kind != gern_pipeline_s::GEMM_F32 && p->kind != gern_pipeline_s::GEMM_BF16) ||
+        A == nullptr || B == nullptr || C == nullptr) {
+        return fail("gern_gemm_run: bad pipeline or null buffer");
+    }
+    if (!p->runner) {
+        return fail("gern_gemm_run: the pipeline was created compile-only");
+    }
+    if (M < 1 || N < 1 || K < 1) {
+        return fail("gern_gemm_run: bad shape");
+    }
+    if (p->kind == gern_pipeline_s::GEMM_BF16 && ((K % 8) != 0 || (N % 2) != 0)) {
+        return fail("gern_gemm_run: the bf16 path needs K % 8 == 0 and N % 2 == 0 (16-byte rows of A, dword pairs of B)");
+    }
+    // MatrixF32 and MatrixBF16 share their layout.
+    hip::MatrixF32 a{static_cast<float *>(const_cast<void *>(A)), M, K, K};
+    hip::MatrixF32 b{static_cast<float *>(const_cast<void *>(B)), K, N, N};
+    hip::MatrixF32 c{C, M, N, N};
+    int64_t k_dim = K;
+    try {
+        p->runner->setStream(stream);
+        p->runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    return 0;
+}
+
+int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_pipeline *out) {
+    if (out == nullptr) {
+        return fail("gern_qk_softmax_create: null argument");
+    }
+    *out = nullptr;
+    if (head_dim < 32 || head_dim > 256 || head_dim % 32 != 0) {
+        return fail("gern_qk_softmax_create: head_dim must be a multiple of 32 in [32, 256]");
+    }
+    if (max_keys < 256 || max_keys > 4096 || max_keys % 256 != 0) {
+        return fail("gern_qk_softmax_create: max_keys must be a multiple of 256 in [256, 4096]");
+    }
+    auto p = std::make_unique<gern_pipeline_s>();
+    p->kind = gern_pipeline_s::QK_SOFTMAX;
+    p->head_dim = head_dim;
+    p->ncol = max_keys;
+    try {
+        auto Q = AbstractDataTypePtr(new const annot::MatrixOperand("Q", annot::MatrixOperand::BF16));
+        auto K = AbstractDataTypePtr(new const annot::MatrixOperand("K", annot::MatrixOperand::BF16));
+        auto S = AbstractDataTypePtr(new const annot::RowBlockF32("S", annot::RowBlockF32::OUTPUT));
+        auto logits = AbstractDataTypePtr(new const annot::RowBlockF32("logits", annot::RowBlockF32::TEMP));
+        auto shifted = AbstractDataTypePtr(new const annot::RowBlockF32("shifted", annot::RowBlockF32::TEMP));
+        auto expd = AbstractDataTypePtr(new const annot::RowBlockF32("expd", annot::RowBlockF32::TEMP));
+        auto row_max = AbstractDataTypePtr(new const annot::RowStat("row_max"));
+        auto row_sum = AbstractDataTypePtr(new const annot::RowStat("row_sum"));
+        Variable rows("rows"), keys("keys"), d("d"), scale("scale", Datatype::Float32), threads("threads");
+        annot::QKScaled qk{Q, K, logits};
+        annot::MaxRow max_row{logits, row_max};
+        annot::SubtractVec sub{row_max, logits, shifted};
+        annot::ExpMatrix ex{shifted, expd};
+        annot::SumRow sum_row{expd, row_sum};
+        annot::DivideVec div{row_sum, expd, S};
+        std::map<std::string, Variable> width{{"ncol", keys.bind(max_keys)}};
+        Composable program = Global(
+            (Tile(S["row"], rows.bind(16)) || Grid::BLOCK_X)(Tile(S["col"], keys.bind(max_keys))(
+                qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), max_row[width](row_max, logits),
+                sub(row_max, logits, shifted), ex(shifted, expd), sum_row[width](row_sum, expd),
+                div(row_sum, expd, S))),
+            {{Grid::BLOCK_DIM_X, threads.bind(256)}});
+        int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
+        if (rc != 0) {
+            return rc;
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    *out = p.release();
+    return 0;
+}
+
+int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M, int64_t N,
+                        float scale, void *stream) {
+    if (p == nullptr || p->kind != gern_pipeline_s::QK_SOFTMAX || Q == nullptr || K == nullptr || S == nullptr) {
+        return fail("gern_qk_softmax_run: bad pipeline or null buffer");
+    }
+    if (!p->runner) {
+        return fail("gern_qk_softmax_run: the pipeline was created compile-only");
+    }
+    if (M < 1 || N < 1 || N > p->ncol) {
+        return fail("gern_qk_softmax_run: N exceeds the max_keys the pipeline was created for");
+    }
+    hip::MatrixF32 q{reinterpret_cast<float *>(const_cast<uint16_t *>(Q)), M, p->head_dim, p->head_dim};
+    hip::MatrixF32 k{reinterpret_cast<float *>(const_cast<uint16_t *>(K)), N, p->head_dim, p->head_dim};
+    hip::MatrixF32 s{S, M, N, N};
+    try {
+        p->runner->setStream(stream);
+        p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"scale", &scale}});
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    return 0;
+}
+
+const char *gern_pipeline_source(gern_pipeline p) {
+    return p ? p->source.c_str() : "";
+}
+
+const char *gern_pipeline_kernel_name(gern_pipeline p) {
+    if (p == nullptr) {
+        return "";
+    }
+    if (p->kernel_name.empty() && p->runner) {
+        p->kernel_name = p->runner->getKernelName();
+    }
+    return p->kernel_name.c_str();
+}
+
+int gern_pipeline_destroy(gern_pipeline p) {
+    delete p;
+    return 0;
+}
+
+size_t gern_pipelines_last_error(char *buf, size_t buf_size) {
+    if (buf != nullptr && buf_size > 0) {
+        size_t n = g_error.size() < buf_size - 1 ? g_error.size() : buf_size - 1;
+        std::memcpy(buf, g_error.data(), n);
+        buf[n] = '\0';
+    }
+    return g_error.size();
+}
+
+}  // extern "C"

@@ -1,0 +1,246 @@
+// Fused S = softmax_rows(scale * Q K^T) for bf16 Q (M x D) and K (N x D).
+//
+// One workgroup (four wavefronts) owns 16 rows of S and ALL N <= 4096 columns,
+// held as MFMA accumulators: wavefront w owns columns [w*N/4, (w+1)*N/4), as
+// N/256 groups of 64 columns, each group four v_mfma_f32_16x16x32_bf16 tiles.
+// Inside a group, tile t / lane column j stands for key 4*j + t, so that the
+// four tiles of a group give every lane FOUR CONSECUTIVE columns of S and a row
+// of the block is stored with 16-byte stores, 256 contiguous bytes per sixteen
+// lanes.  The logits never leave registers: row maximum and row sum are reduced
+// inside the 16-lane DPP rows that share an S row, then across the four
+// wavefronts through 256 bytes of LDS.  S is written once; Q and K (1 MiB each,
+// L2-resident) are the only reads.
+//
+// The reference has nothing like this (no bf16, no matrix-core path, no fused
+// GEMM -> softmax); the softmax stages reuse the names and argument order of
+// its softmax gernels (apps/common/impl/impl.h:7-188) so that the same
+// annotations compose them.
+#pragma once
+
+#include "gernels/mm.h"
+#include "gernels/softmax.h"
+
+namespace gernels {
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 x N logits / probabilities, distributed over the workgroup as described
+// above: acc[g][t][i] is row 4*(lane/16) + i, column
+// wave*(N/4) + 64*g + 4*(lane%16) + t.
+template<int64_t R, int64_t N>
+struct RowBlock {
+    static_assert(R == 16, "a row block is one MFMA tile high");
+    static_assert(N % 256 == 0 && N <= 4096, "four wavefronts x 64-column groups, at most 256 accumulators");
+    static constexpr int64_t rows = R;
+    static constexpr int64_t cols = N;
+    static constexpr int G = (int)(N / 256);
+    f32x4_t acc[G][4];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+// Per-row scalars of a row block: lane l keeps rows 4*(l/16) .. +3.
+template<int64_t R>
+struct RowStat {
+    static constexpr int64_t size = R;
+    float v[4];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+template<int64_t R, int64_t N>
+__device__ __forceinline__ RowBlock<R, N> allocate_row_block() {
+    return RowBlock<R, N>();
+}
+
+template<int64_t R>
+__device__ __forceinline__ RowStat<R> allocate_row_stat() {
+    return RowStat<R>();
+}
+
+// The output window of a row block (nothing is read).
+template<int64_t R, int64_t N>
+__device__ __forceinline__ RowBlock<R, N> MatrixF32::view_row_block(int64_t, int64_t) const {
+    return RowBlock<R, N>();
+}
+
+template<int64_t R, int64_t N>
+__device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y, const RowBlock<R, N> &t) const {
+    const int lane = lane_id();
+    const int w = (int)(threadIdx.x / kWaveSize);
+    const int64_t c0 = y + (int64_t)w * (N / 4) + 4 * (lane % 16);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int64_t rr = x + 4 * (lane / 16) + i;
+        if (rr >= row) {
+            continue;
+        }
+        float *p = data + rr * lda;
+        const bool vec_ok = ((((uint64_t)(p + y)) & 15u) == 0);
+#pragma unroll
+        for (int g = 0; g < RowBlock<R, N>::G; g++) {
+            const int64_t cc = c0 + 64 * g;
+            const float4 val = make_float4(t.acc[g][0][i], t.acc[g][1][i], t.acc[g][2][i], t.acc[g][3][i]);
+            if (vec_ok && cc + 3 < col) {
+                *reinterpret_cast<float4 *>(p + cc) = val;
+            } else {
+                if (cc + 0 < col) p[cc + 0] = val.x;
+                if (cc + 1 < col) p[cc + 1] = val.y;
+                if (cc + 2 < col) p[cc + 2] = val.z;
+                if (cc + 3 < col) p[cc + 3] = val.w;
+            }
+        }
+    }
+}
+
+// S = scale * Q K^T for the 16 rows of Q in view; columns past the last key
+// get -inf so that they vanish from the softmax.
+template<int64_t R, int64_t N, int64_t D>
+__device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t> &Q, const GlobalView<N, D, uint16_t> &K,
+                                          RowBlock<R, N> &S, float scale) {
+    static_assert(D % 32 == 0 && D <= 256, "head dimension in MFMA K steps of 32");
+    constexpr int KS = (int)(D / 32);
+    const int lane = lane_id();
+    const int w = (int)(threadIdx.x / kWaveSize);
+    const int k_off = 8 * (lane / 16);
+
+    bf16x8_t q[KS];
+    {
+        const int64_t r = lane % 16;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (r < Q.rows) {
+                v = *reinterpret_cast<const uint4 *>(Q.data + r * Q.lda + s * 32 + k_off);
+            }
+            q[s] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < RowBlock<R, N>::G; g++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int64_t key = (int64_t)w * (N / 4) + 64 * g + 4 * (lane % 16) + t;
+            const bool ok = key < K.rows;
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                uint4 v = make_uint4(0u, 0u, 0u, 0u);
+                if (ok) {
+                    v = *reinterpret_cast<const uint4 *>(K.data + key * K.lda + s * 32 + k_off);
+                }
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(q[s], __builtin_bit_cast(bf16x8_t, v), acc, 0, 0, 0);
+            }
+            S.acc[g][t] = acc * scale;
+        }
+        // The column a lane holds in tile t is its own key, so validity is a
+        // per-lane, per-tile property.
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int64_t key = (int64_t)w * (N / 4) + 64 * g + 4 * (lane % 16) + t;
+            if (key >= K.rows) {
+                S.acc[g][t] = f32x4_t{-__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf(),
+                                      -__builtin_huge_valf()};
+            }
+        }
+    }
+}
+
+namespace detail {
+
+// Reduces over the 16 lanes of a DPP row (the lanes that share S rows), then
+// over the four wavefronts.
+template<typename Op>
+__device__ __forceinline__ float row_block_reduce(float x, float *lds, int slot) {
+    x = Op::apply(x, dpp_move<0xB1>(x));   // quad_perm [1,0,3,2]
+    x = Op::apply(x, dpp_move<0x4E>(x));   // quad_perm [2,3,0,1]
+    x = Op::apply(x, dpp_move<0x141>(x));  // row_half_mirror
+    x = Op::apply(x, dpp_move<0x140>(x));  // row_mirror
+    const int w = (int)(threadIdx.x / kWaveSize);
+    lds[w * 16 + slot] = x;  // all 16 lanes of the row write the same value
+    __syncthreads();
+    float r = Op::apply(Op::apply(lds[slot], lds[16 + slot]), Op::apply(lds[32 + slot], lds[48 + slot]));
+    __syncthreads();
+    return r;
+}
+
+template<typename Op, int64_t R, int64_t N>
+__device__ __forceinline__ void reduce_row_block(RowStat<R> &out, const RowBlock<R, N> &in) {
+    __shared__ float scratch[64];
+    const int lane = lane_id();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float acc = Op::identity();
+#pragma unroll
+        for (int g = 0; g < RowBlock<R, N>::G; g++) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                acc = Op::apply(acc, in.acc[g][t][i]);
+            }
+        }
+        out.v[i] = row_block_reduce<Op>(acc, scratch, 4 * (lane / 16) + i);
+    }
+}
+
+}  // namespace detail
+
+template<int64_t stride = 64, int64_t R, int64_t N>
+__device__ __forceinline__ void max_row(RowStat<R> &out, const RowBlock<R, N> &in) {
+    detail::reduce_row_block<MaxOp>(out, in);
+}
+
+template<int64_t stride = 64, int64_t R, int64_t N>
+__device__ __forceinline__ void sum_row(RowStat<R> &out, const RowBlock<R, N> &in) {
+    detail::reduce_row_block<SumOp>(out, in);
+}
+
+template<int64_t R, int64_t N>
+__device__ __forceinline__ void subtract_vec(const RowStat<R> &vec, const RowBlock<R, N> &in, RowBlock<R, N> &out) {
+#pragma unroll
+    for (int g = 0; g < RowBlock<R, N>::G; g++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out.acc[g][t][i] = in.acc[g][t][i] - vec.v[i];
+            }
+        }
+    }
+}
+
+template<int64_t R, int64_t N>
+__device__ __forceinline__ void exp_matrix(const RowBlock<R, N> &in, RowBlock<R, N> &out) {
+#pragma unroll
+    for (int g = 0; g < RowBlock<R, N>::G; g++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out.acc[g][t][i] = expf(in.acc[g][t][i]);
+            }
+        }
+    }
+}
+
+template<int64_t R, int64_t N>
+__device__ __forceinline__ void divide_vec(const RowStat<R> &vec, const RowBlock<R, N> &in, RowBlock<R, N> &out) {
+    float rcp[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        rcp[i] = 1.0f / vec.v[i];
+    }
+#pragma unroll
+    for (int g = 0; g < RowBlock<R, N>::G; g++) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out.acc[g][t][i] = div_by(in.acc[g][t][i], vec.v[i], rcp[i]);
+            }
+        }
+    }
+}
+
+}  // namespace gernels

@@ -50,6 +50,18 @@ __device__ __forceinline__ WaveVec<R> allocate_wave_vec() {
     return WaveVec<R>();
 }
 
+// Defined in gernels/mm.h: a window onto a matrix in HBM (no data movement) and
+// the two block-distributed accumulator tiles of the GEMM gernels.
+template<int64_t R, int64_t C, typename T>
+struct GlobalView;
+template<int64_t BM, int64_t BN>
+struct MfmaAcc;
+template<int64_t BM, int64_t BN>
+struct FmaAcc;
+// Defined in gernels/qk_softmax.h: sixteen full rows of logits in registers.
+template<int64_t R, int64_t N>
+struct RowBlock;
+
 // Row-major fp32 matrix in HBM.  Plain aggregate: the host fills one in and
 // the launch passes it by value, so host and device layouts must agree
 // (pointer, then three 64-bit integers).
@@ -58,6 +70,23 @@ struct MatrixF32 {
     int64_t row;
     int64_t col;
     int64_t lda;
+
+    // GEMM operand / result access (gernels/mm.h).
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ GlobalView<R, C, float> view(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ MfmaAcc<BM, BN> load_acc_mfma(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN> &t) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ FmaAcc<BM, BN> load_acc_fma(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const;
+    // Fused QK^T -> softmax result access (gernels/qk_softmax.h).
+    template<int64_t R, int64_t N>
+    __device__ __forceinline__ RowBlock<R, N> view_row_block(int64_t x, int64_t y) const;
+    template<int64_t R, int64_t N>
+    __device__ __forceinline__ void store_row_block(int64_t x, int64_t y, const RowBlock<R, N> &t) const;
 
     // Loads the R x C tile whose top-left element is (x, y).  Elements outside
     // the matrix read as 0; a tile may therefore hang over the right or bottom

@@ -480,9 +480,21 @@ struct less<gern::ADTMember> {
 };
 template<>
 struct less<gern::Expr> {
+    // Variables order by name and members by (structure, member), so that a
+    // loop bound is found no matter which handle of it the user passes; every
+    // other expression orders by node identity.
     bool operator()(const gern::Expr &a, const gern::Expr &b) const {
-        const bool am = gern::isa<gern::ADTMember>(a), bm = gern::isa<gern::ADTMember>(b);
-        if (am && bm) {
+        auto rank = [](const gern::Expr &e) {
+            return gern::isa<gern::Variable>(e) ? 0 : gern::isa<gern::ADTMember>(e) ? 1 : 2;
+        };
+        const int ra = rank(a), rb = rank(b);
+        if (ra != rb) {
+            return ra < rb;
+        }
+        if (ra == 0) {
+            return std::less<gern::Variable>()(gern::to<gern::Variable>(a), gern::to<gern::Variable>(b));
+        }
+        if (ra == 1) {
             return std::less<gern::ADTMember>()(gern::to<gern::ADTMember>(a), gern::to<gern::ADTMember>(b));
         }
         return a.ptr < b.ptr;

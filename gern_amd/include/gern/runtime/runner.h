@@ -63,6 +63,12 @@ public:
     std::vector<std::string> getArgumentOrder() const {
         return argument_order;
     }
+    // Device launches: the instantiated kernel's name expression, and the HIP
+    // stream later evaluate() calls launch on.
+    std::string getKernelName() const;
+    void setStream(void *s) {
+        stream = s;
+    }
 
 private:
     FunctionSignature signature;

@@ -237,7 +237,7 @@ void Computation::infer_relationships(AbstractDataTypePtr output, std::vector<Va
         // A structure read by several later stages: every reader is assumed to
         // need the same subset, and the first reader (in program order)
         // defines it.
-        std::cout << "WARNING::FORKS ARE NOT IMPL, ASSUMING EQUAL CONSUMPTION!" << std::endl;
+        std::cerr << "WARNING::FORKS ARE NOT IMPL, ASSUMING EQUAL CONSUMPTION!" << std::endl;
     }
     const Composable &consumer = it->second.front();
     std::vector<Expr> needed = consumer.getAnnotation().getPattern().getRequirement(output);

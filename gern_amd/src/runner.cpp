@@ -197,6 +197,10 @@ std::string Runner::getSource() const {
     return source;
 }
 
+std::string Runner::getKernelName() const {
+    return plan ? plan->name_expression : std::string();
+}
+
 void evaluate(Composable c, std::map<std::string, void *> args, Runner::Options config) {
     Runner runner(c);
     runner.compile(config);

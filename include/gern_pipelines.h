@@ -1,0 +1,90 @@
+/*
+ * gern_pipelines.h - C ABI over the fused pipelines of the hot path.
+ *
+ * Each *_create call does what the `main()` of the corresponding reference
+ * application does with Gern's C++ API: declare the data structures, compose
+ * the annotated functions with Tile / Reduce / Global, hand the program to a
+ * Runner and compile it (here: HIP for gfx950 through hiprtc).  Each *_run
+ * call is Runner::evaluate on caller-owned DEVICE buffers; it is asynchronous
+ * on the given HIP stream (NULL = default stream).
+ *
+ * Plain pointers and sizes only.  Every function returns 0 on success; on
+ * failure the calling thread's message is read with gern_pipelines_last_error().
+ * A failure to find a GPU is an error, never a fallback.
+ */
+#ifndef GERN_PIPELINES_H
+#define GERN_PIPELINES_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gern_pipeline_s *gern_pipeline;
+
+enum {
+    /* Generate the source and compile it for gfx950, but do not load it: the
+     * pipeline can be inspected (gern_pipeline_source) on a machine without a
+     * GPU and cannot be run. */
+    GERN_PIPELINE_COMPILE_ONLY = 1,
+    /* Launch workgroups in plain blockIdx order (no XCD-aware renumbering). */
+    GERN_PIPELINE_NO_XCD_REMAP = 2
+};
+
+/* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
+ * applied left to right ("xy" = horizontal then vertical, "xyx" = the
+ * three-stage chain); every stage has `stride` taps of weight 1/stride and
+ * produces the valid region only.  One wavefront produces one
+ * tile_rows x tile_cols output tile; tile_cols + (#x stages)*(stride-1) must
+ * not exceed 256.  waves_per_block wavefronts (side by side along the
+ * columns) form a workgroup.
+ * Composes what apps/blur/blur.cpp:31-73 composes (there: blur_x, blur_y). */
+int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_rows, int64_t tile_cols,
+                           int waves_per_block, int flags, gern_pipeline *out);
+/* in is rows x cols (row stride ld_in); out is
+ * (rows - ny*(stride-1)) x (cols - nx*(stride-1)) (row stride ld_out).
+ * Runner::evaluate of the program above, apps/blur/blur.cpp:85-88. */
+int gern_blur_chain_run(gern_pipeline p, const float *in, int64_t rows, int64_t cols, int64_t ld_in,
+                        float *out, int64_t ld_out, void *stream);
+
+/* Row-wise numerically stable softmax over matrices with exactly `ncol`
+ * columns: max, x - max, exp, sum, divide, fused; rows_per_wave rows are held
+ * in registers by one wavefront.  The five calls are the reference's softmax
+ * gernels, apps/common/annot/functions.h:9-173. */
+int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pipeline *out);
+int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows, int64_t ld,
+                     void *stream);
+
+/* Dense GEMM C += A * B, row-major, A is M x K, B is K x N, C is M x N fp32.
+ * variant 0: fp32 inputs, vector-ALU FMAs.
+ * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA.
+ * Composes Tile(i)(Tile(j)(Reduce(k)(matrix_multiply))) as
+ * gernels/mm/kernel_3.cu:61-75 does. */
+int gern_gemm_create(int variant, int flags, gern_pipeline *out);
+int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64_t M, int64_t N,
+                  int64_t K, void *stream);
+
+/* S = softmax_rows(scale * Q K^T): Q is M x D and K is N x D in bf16 (bit
+ * patterns), S is M x N fp32; MFMA tiles feed an in-register row reduction.
+ * head_dim = D (a multiple of 32, at most 256); max_keys bounds N (a multiple
+ * of 256, at most 4096: sixteen rows of logits stay in accumulators).
+ * No counterpart in the reference (it has no bf16 and no matrix-core path);
+ * the softmax stages are those of apps/common/annot/functions.h:9-173. */
+int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_pipeline *out);
+int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M,
+                        int64_t N, float scale, void *stream);
+
+/* The generated device source (owned by the pipeline, valid until destroy). */
+const char *gern_pipeline_source(gern_pipeline p);
+/* The name expression of the instantiated kernel, e.g. "function_7<252, 8, 3>". */
+const char *gern_pipeline_kernel_name(gern_pipeline p);
+int gern_pipeline_destroy(gern_pipeline p);
+
+size_t gern_pipelines_last_error(char *buf, size_t buf_size);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,88 @@
+"""The C ABI libraries load and export every symbol the headers declare, and
+the pipelines generate HIP that compiles for gfx950.  No GPU, no compute."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import gern_amd
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gern_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_runtime_abi_exports_every_declared_symbol():
+    hip = gern_amd.hip_lib()
+    names = _declared("gern_hip.h")
+    assert len(names) >= 20
+    missing = [n for n in names if not hasattr(hip, n)]
+    assert not missing, missing
+
+
+def test_pipeline_abi_exports_every_declared_symbol():
+    pipes = gern_amd.pipelines_lib()
+    names = _declared("gern_pipelines.h")
+    assert len(names) >= 10
+    missing = [n for n in names if not hasattr(pipes, n)]
+    assert not missing, missing
+
+
+def test_blur_chain_generates_fused_kernel_with_inferred_halos():
+    p = gern_amd.BlurChain("xyx", tile_rows=8, flags=gern_amd.COMPILE_ONLY)
+    src = p.source
+    assert p.kernel_name.endswith("<252, 8, 3, 64>")
+    assert src.count("__global__") == 1 and "__launch_bounds__(64)" in src
+    # input tile: (row + 2) x (col + 4); first temporary (row + 2) x (col + 2)
+    assert "load_wave<((row + stride) - 1), ((((col + stride) - 1) + stride) - 1)>" in src
+    assert "allocate_wave_tile<((row + stride) - 1), ((col + stride) - 1)>" in src
+    assert "allocate_wave_tile<row, ((col + stride) - 1)>" in src
+    assert src.index("blur_x<stride>") < src.index("blur_y<stride>") < src.rindex("blur_x<stride>")
+    assert "gern_block_x" in src  # XCD-aware workgroup order
+
+
+def test_blur_chain_wavefront_mapping_and_plain_order():
+    p = gern_amd.BlurChain("xy", tile_rows=4, waves_per_block=4, flags=gern_amd.COMPILE_ONLY | gern_amd.NO_XCD_REMAP)
+    src = p.source
+    assert "(threadIdx.x / 64)" in src and "__launch_bounds__(256)" in src
+    assert "gern_block_x" not in src and "blockIdx.x" in src
+
+
+def test_softmax_generates_one_pass_kernel():
+    p = gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY)
+    src = p.source
+    for fn in ("max_row", "subtract_vec", "exp_matrix", "sum_row", "divide_vec"):
+        assert "gernels::" + fn in src
+    assert src.count("load_wave") == 1  # the row is read once
+
+
+def test_bad_arguments_are_errors():
+    with pytest.raises(gern_amd.GernError, match="pattern"):
+        gern_amd.BlurChain("xz", flags=gern_amd.COMPILE_ONLY)
+    with pytest.raises(gern_amd.GernError, match="tile_cols"):
+        gern_amd.BlurChain("xyx", tile_cols=256, flags=gern_amd.COMPILE_ONLY)
+    with pytest.raises(gern_amd.GernError):
+        gern_amd.Softmax(100000, flags=gern_amd.COMPILE_ONLY)
+
+
+def test_compile_only_pipeline_refuses_to_run():
+    p = gern_amd.Softmax(256, flags=gern_amd.COMPILE_ONLY)
+    rc = gern_amd.pipelines_lib().gern_softmax_run(p.h, C.c_void_p(16), C.c_void_p(16), 1, 256, None)
+    assert rc != 0
+
+
+def test_runtime_reports_compile_errors():
+    hip = gern_amd.hip_lib()
+    src = b"__global__ void broken( { }"
+    names = (C.c_char_p * 1)(b"broken")
+    size = C.c_size_t()
+    rc = hip.gern_hip_compile_only(src, names, 1, None, 0, b"gfx950", C.byref(size))
+    assert rc == 1
+    buf = C.create_string_buffer(4096)
+    hip.gern_hip_last_error(buf, 4096)
+    assert b"error" in buf.value
