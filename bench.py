@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-kernel hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only NAME]
+
+A step is one launch of the fused three-stage blur chain (x, y, x; 3 taps of
+weight 1/3) on an 8192 x 8192 fp32 image that is already resident in HBM; the
+headline value is its whole-job throughput in GB/s of ALGORITHMIC bytes
+(logical input read once + logical output written once).  The same line also
+carries the other configurations of the metric (row softmax, GEMM fp32 / bf16,
+fused QK^T softmax), each with its own roofline fraction, a roofline object
+for the dominant kernel timed with HIP events on the launching stream, and the
+CPU baseline: the reference library's own CPU lowering of the same composed
+pipeline (oracle/_ref/, when it was built) or the CPU oracle, timed on one host
+core.
+
+Prints exactly one JSON line on stdout.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA
+FP32_VECTOR_PEAK_TFLOPS = 157.3
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_launches(fn, warmup, steps, torch, gern_amd):
+    """Returns (wall ms per step, event ms per step) over exactly `steps` launches."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = gern_amd.Event(), gern_amd.Event()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, start.elapsed_ms_until(stop) / steps
+
+
+def cpu_baseline_blur(img_np):
+    """The same composed pipeline on ONE host core."""
+    from oracle import oracle as o
+    from oracle import ref
+    rows, cols = img_np.shape
+    if ref.available():
+        kind = "reference"
+        # tile sizes must divide the 8190 x 8188 output (the reference handles no ragged tiles)
+        run = lambda: ref.blur_chain(img_np, "xyx", 90, 356)  # noqa: E731
+        what = "reference library CPU lowering of Tile(rows=90)(Tile(cols=356)(blur_x, blur_y, blur_x)), g++ -O2"
+    else:
+        kind = "port"
+        run = lambda: o.blur_chain_tiled(img_np, "xyx", 90, 356)  # noqa: E731
+        what = "CPU oracle (scalar C restatement), same tiling, gcc -O2"
+    run()  # warm-up
+    times = []
+    budget = time.perf_counter() + 20.0
+    while len(times) < 5 and (len(times) < 1 or time.perf_counter() < budget):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    nbytes = rows * cols * 4 + (rows - 2) * (cols - 4) * 4
+    return {
+        "value": nbytes / med / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "host_cores": os.cpu_count(),
+        "kind": kind,
+        "seconds": med,
+        "sample": "full workload (8192x8192 three-stage blur), median of %d runs after one warm-up; %s" % (len(times), what),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="run only this workload (blur, softmax, gemm_f32, gemm_bf16, qk_softmax)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import numpy as np
+    import torch
+
+    import gern_amd
+    from gern_amd import inputs
+
+    if gern_amd.device_count() < 1 or not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: there is no CPU fallback")
+    lim = gern_amd.device_limits()
+    log("device:", lim.arch.decode(), "CUs:", lim.compute_units)
+
+    want = lambda name: (not args.only) or args.only == name  # noqa: E731
+    workloads = {}
+    result = None
+
+    # ---- config 2: three-stage blur, 8192 x 8192 (the headline) ------------
+    if want("blur"):
+        rows = cols = 8192
+        img = inputs.uniform((rows, cols), 2)
+        d_in = torch.from_numpy(img).cuda()
+        blur = gern_amd.BlurChain("xyx", tile_rows=4)
+        d_out = torch.zeros(blur.out_shape(rows, cols), device="cuda")
+        wall, ev = time_launches(lambda: blur(d_in, d_out), args.warmup, args.steps, torch, gern_amd)
+        nbytes = img.nbytes + d_out.numel() * 4
+        gbs = nbytes / (wall * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": nbytes / (ev * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                "kernel": blur.kernel_name, "kernel_ms": ev, "algorithmic_bytes": nbytes}
+        workloads["blur_xyx_8192"] = {"GB/s": gbs, "ms": wall, "frac_hbm": gbs / HBM_PEAK_GBS}
+        log("blur xyx 8192^2: %.1f us/launch  %.0f GB/s  (%.1f%% of HBM peak)" % (wall * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
+        result = {
+            "metric": "fused 3-stage blur (x,y,x) 8192x8192 fp32, algorithmic GB/s",
+            "value": gbs,
+            "unit": "GB/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": wall,
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "f32",
+            "data": "synthetic",
+            "config": {"workload": "three-stage fused separable blur chain (3-tap x, y, x; weights 1/3), 8192x8192 fp32 "
+                                   "uniform[0,1) seed 2, valid-region output 8190x8188, one launch per step",
+                       "schedule": "one wavefront per 4x252 output tile, XCD-aware workgroup order"},
+            "roofline": roof,
+        }
+        if not args.no_cpu:
+            result["cpu_baseline"] = cpu_baseline_blur(img)
+            log("cpu baseline: %.2f GB/s on 1 core (%s)" % (result["cpu_baseline"]["value"], result["cpu_baseline"]["kind"]))
+        del d_in, d_out
+
+    steps2 = max(10, args.steps // 4)
+    # ---- config 3: row softmax, 8192 x 4096 --------------------------------
+    if want("softmax"):
+        x = inputs.normal((8192, 4096), 3, 0.0, 2.0)
+        d_x = torch.from_numpy(x).cuda()
+        d_y = torch.zeros_like(d_x)
+        sm = gern_amd.Softmax(4096)
+        wall, ev = time_launches(lambda: sm(d_x, d_y), args.warmup, steps2, torch, gern_amd)
+        gbs = 2 * x.nbytes / (ev * 1e-3) / 1e9
+        workloads["softmax_8192x4096"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "kernel": sm.kernel_name}
+        log("softmax 8192x4096: %.1f us  %.0f GB/s (%.1f%%)" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
+        del d_x, d_y
+
+    # ---- config 4: GEMM 4096^3 ---------------------------------------------
+    for variant, peak in (("f32", FP32_VECTOR_PEAK_TFLOPS), ("bf16", MFMA_BF16_PEAK_TFLOPS)):
+        if not want("gemm_" + variant):
+            continue
+        n = 4096
+        A = inputs.uniform((n, n), 4, -1.0, 1.0)
+        B = inputs.uniform((n, n), 5, -1.0, 1.0)
+        if variant == "bf16":
+            dA = torch.from_numpy(inputs.to_bf16_bits(A).view(np.int16)).cuda()
+            dB = torch.from_numpy(inputs.to_bf16_bits(B).view(np.int16)).cuda()
+        else:
+            dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+        dC = torch.zeros((n, n), device="cuda")
+        g = gern_amd.Gemm(variant)
+        wall, ev = time_launches(lambda: g(dA, dB, dC), 3, max(5, args.steps // 20), torch, gern_amd)
+        tf = 2.0 * n ** 3 / (ev * 1e-3) / 1e12
+        workloads["gemm_%s_4096" % variant] = {"TFLOP/s": tf, "ms": ev, "frac_peak": tf / peak, "peak_TFLOP/s": peak,
+                                               "kernel": g.kernel_name}
+        log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, ev * 1e3, tf, 100 * tf / peak, peak))
+        del dA, dB, dC
+
+    # ---- config 5: fused QK^T -> softmax ------------------------------------
+    if want("qk_softmax"):
+        m = nk = 4096
+        d = 128
+        Q = inputs.to_bf16_bits(inputs.normal((m, d), 5))
+        K = inputs.to_bf16_bits(inputs.normal((nk, d), 6))
+        dQ = torch.from_numpy(Q.view(np.int16)).cuda()
+        dK = torch.from_numpy(K.view(np.int16)).cuda()
+        dS = torch.zeros((m, nk), device="cuda")
+        qk = gern_amd.QKSoftmax(d, nk)
+        scale = 1.0 / np.sqrt(float(d))
+        wall, ev = time_launches(lambda: qk(dQ, dK, dS, scale), args.warmup, steps2, torch, gern_amd)
+        nbytes = Q.nbytes + K.nbytes + m * nk * 4
+        gbs = nbytes / (ev * 1e-3) / 1e9
+        tf = 2.0 * m * nk * d / (ev * 1e-3) / 1e12
+        workloads["qk_softmax_4096x4096x128"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "TFLOP/s": tf,
+                                                 "frac_mfma": tf / MFMA_BF16_PEAK_TFLOPS, "kernel": qk.kernel_name}
+        log("qk softmax 4096x4096x128: %.1f us  %.0f GB/s (%.1f%% HBM)  %.1f TFLOP/s" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS, tf))
+
+    if result is None:
+        result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "", "n_gpus": 1,
+                  "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
+                  "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": args.only}}
+    result["workloads"] = workloads
+    result["device"] = {"arch": lim.arch.decode(), "compute_units": lim.compute_units, "clock_khz": lim.clock_khz}
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

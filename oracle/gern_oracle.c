@@ -374,7 +374,11 @@ float oracle_div_const_fma(float x, float d) {
     const float c = 1.0f / d;
     float q = x * c;
     float r = fmaf(-d, q, x);
-    return fmaf(r, c, q);
+    q = fmaf(r, c, q);
+    /* The device code finishes with v_div_fixup_f32, which returns the IEEE
+     * result for zero, infinite and NaN operands (sign of a zero included). */
+    if (x == 0.0f || isinf(x) || x != x) return x / d;
+    return q;
 }
 
 uint64_t oracle_div_const_mismatches(float d, uint32_t lo_bits, uint32_t hi_bits) {

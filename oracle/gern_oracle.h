@@ -99,8 +99,9 @@ void oracle_qk_softmax_rows(const uint16_t *Q, const uint16_t *Kmat, float *S, i
                             int64_t N, int64_t D, float scale, int64_t i0, int64_t i1);
 
 /* ---- division by a constant ------------------------------------------- */
-/* q = x * RN(1/d); r = fma(-d, q, x); q' = fma(r, RN(1/d), q).  The HIP blur
- * gernels divide this way; this restates it with libm fmaf. */
+/* q = x * RN(1/d); r = fma(-d, q, x); q' = fma(r, RN(1/d), q), then the IEEE
+ * result for zero / infinite / NaN dividends (what v_div_fixup_f32 does).  The
+ * HIP blur gernels divide this way; this restates it with libm fmaf. */
 float oracle_div_const_fma(float x, float d);
 /* Number of fp32 bit patterns in [lo_bits, hi_bits) for which
  * oracle_div_const_fma(x,d) differs bitwise from x / d (NaNs skipped). */
