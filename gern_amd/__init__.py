@@ -17,6 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 COMPILE_ONLY = 1
 NO_XCD_REMAP = 2
+GEMM_OVERWRITE = 4
 
 _libs = None
 
@@ -212,11 +213,14 @@ class Softmax(_Pipeline):
 
 
 class Gemm(_Pipeline):
-    """C += A @ B.  variant "f32" (vector ALU) or "bf16" (MFMA, fp32 accumulate)."""
+    """C += A @ B (or C = A @ B with overwrite=True).  variant "f32" (vector
+    ALU) or "bf16" (MFMA, fp32 accumulate)."""
 
-    def __init__(self, variant="f32", flags=0):
+    def __init__(self, variant="f32", overwrite=False, flags=0):
         super().__init__()
         self.variant = variant
+        if overwrite:
+            flags |= GEMM_OVERWRITE
         _check(pipelines_lib().gern_gemm_create({"f32": 0, "bf16": 1}[variant], flags, C.byref(self.h)))
 
     def __call__(self, A, B, Cm, stream=None):

@@ -15,8 +15,10 @@ namespace annot {
 class MatrixOperand : public AbstractDataType {
 public:
     enum Element { F32, BF16 };
-    MatrixOperand(const std::string &name, Element element)
-        : name(name), element(element) {
+    // exact: the caller guarantees that the matrix extents are multiples of
+    // the window sizes the program tiles with, so windows need no bounds tests.
+    MatrixOperand(const std::string &name, Element element, bool exact = false)
+        : name(name), element(element), exact(exact) {
     }
     std::string getName() const override {
         return name;
@@ -38,7 +40,7 @@ public:
     }
     FunctionSignature getQueryFunction() const override {
         return FunctionSignature{
-            .name = "template view",
+            .name = exact ? "template view_exact" : "template view",
             .args = {x, y},
             .template_args = {row, col},
         };
@@ -51,6 +53,7 @@ public:
 private:
     std::string name;
     Element element;
+    bool exact;
     Variable x{"x"};
     Variable y{"y"};
     Variable row{"row", Datatype::Int64, true};
@@ -58,12 +61,16 @@ private:
 };
 
 // The GEMM result in HBM; its subsets are block-distributed accumulator tiles
-// (loaded from C, so the product is added to what C holds, and stored back).
+// that start at zero and are either ADDED to C when inserted (accumulate: the
+// reference's C += A * B) or written over it (C = A * B; C is never read).
+//   FMA    fp32 FMAs, 256 threads
+//   MFMA4  matrix cores, four wavefronts (any shape)
+//   MFMA8  matrix cores, eight wavefronts (the fast shape)
 class MatrixAccumulator : public AbstractDataType {
 public:
-    enum Engine { FMA, MFMA };
-    MatrixAccumulator(const std::string &name, Engine engine)
-        : name(name), engine(engine) {
+    enum Engine { FMA, MFMA4, MFMA8 };
+    MatrixAccumulator(const std::string &name, Engine engine, bool accumulate = true)
+        : name(name), engine(engine), accumulate(accumulate) {
     }
     std::string getName() const override {
         return name;
@@ -82,13 +89,15 @@ public:
     }
     FunctionSignature getInsertFunction() const override {
         return FunctionSignature{
-            .name = "store_acc",
+            .name = accumulate ? "add_acc" : "store_acc",
             .args = {x, y},
         };
     }
     FunctionSignature getQueryFunction() const override {
         return FunctionSignature{
-            .name = engine == MFMA ? "template load_acc_mfma" : "template load_acc_fma",
+            .name = engine == MFMA8   ? "template load_acc_mfma8" :
+                    engine == MFMA4 ? "template load_acc_mfma" :
+                                      "template load_acc_fma",
             .args = {x, y},
             .template_args = {row, col},
         };
@@ -103,6 +112,7 @@ public:
 private:
     std::string name;
     Engine engine;
+    bool accumulate;
     Variable x{"x"};
     Variable y{"y"};
     Variable row{"row", Datatype::Int64, true};

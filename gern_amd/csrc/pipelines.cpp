@@ -49,6 +49,7 @@ AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
 struct gern_pipeline_s {
     enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
+    std::unique_ptr<Runner> exact;   // GEMM bf16: the kernel for shapes that are multiples of the tile
     std::string source;
     std::string kernel_name;
     // blur
@@ -262,6 +263,24 @@ int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows,
     return 0;
 }
 
+namespace {
+
+// Tile(i)(Tile(j)(Reduce(k)(matrix_multiply))) for one choice of data
+// structures; one call of the gernel walks a whole 4096-deep K chunk.
+Composable gemmProgram(annot::MatrixOperand::Element element, bool exact, annot::MatrixAccumulator::Engine engine,
+                       bool accumulate, int64_t bm, int64_t bn, int64_t threads_per_block, int64_t lds) {
+    auto A = AbstractDataTypePtr(new const annot::MatrixOperand("A", element, exact));
+    auto B = AbstractDataTypePtr(new const annot::MatrixOperand("B", element, exact));
+    auto C = AbstractDataTypePtr(new const annot::MatrixAccumulator("C", engine, accumulate));
+    Variable ti("ti"), tj("tj"), tk("tk"), k_dim("k_dim"), threads("threads"), smem("smem");
+    annot::MatrixMultiply mm{A, B, C};
+    return Global((Tile(C["row"], ti.bind(bm)) || Grid::BLOCK_Y)((Tile(C["col"], tj.bind(bn)) || Grid::BLOCK_X)(
+                      Reduce(k_dim, tk.bind(4096))(mm[{{"k_dim", k_dim}}](A, B, C)))),
+                  {{Grid::BLOCK_DIM_X, threads.bind(threads_per_block)}}, smem.bind(lds));
+}
+
+}  // namespace
+
 int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
     if (out == nullptr) {
         return fail("gern_gemm_create: null argument");
@@ -272,26 +291,34 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
     }
     auto p = std::make_unique<gern_pipeline_s>();
     p->kind = variant == 1 ? gern_pipeline_s::GEMM_BF16 : gern_pipeline_s::GEMM_F32;
+    const bool accumulate = !(flags & GERN_PIPELINE_GEMM_OVERWRITE);
     try {
-        const bool mfma = variant == 1;
-        // Workgroup tile and the LDS its two pipeline stages need
-        // (gernels/mm.h: mfma_lds_bytes / fma_lds_bytes).
-        const int64_t bm = mfma ? 128 : 128, bn = mfma ? 128 : 128;
-        const int64_t lds = mfma ? 2 * (bm + bn) * 144 : 2 * 2 * 16 * 132 * 4;
-        auto A = AbstractDataTypePtr(new const annot::MatrixOperand(
-            "A", mfma ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32));
-        auto B = AbstractDataTypePtr(new const annot::MatrixOperand(
-            "B", mfma ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32));
-        auto C = AbstractDataTypePtr(new const annot::MatrixAccumulator(
-            "C", mfma ? annot::MatrixAccumulator::MFMA : annot::MatrixAccumulator::FMA));
-        Variable ti("ti"), tj("tj"), tk("tk"), k_dim("k_dim"), threads("threads"), smem("smem");
-        annot::MatrixMultiply mm{A, B, C};
-        // One call walks a whole 4096-deep K chunk, pipelined inside the gernel.
-        Composable program = Global(
-            (Tile(C["row"], ti.bind(bm)) || Grid::BLOCK_Y)((Tile(C["col"], tj.bind(bn)) || Grid::BLOCK_X)(
-                Reduce(k_dim, tk.bind(4096))(mm[{{"k_dim", k_dim}}](A, B, C)))),
-            {{Grid::BLOCK_DIM_X, threads.bind(256)}}, smem.bind(lds));
-        int rc = finish(p.get(), program, flags);
+        int rc;
+        if (variant == 1) {
+            // LDS of the two pipeline stages: gernels/mm.h, mfma_lds_bytes().
+            const int64_t lds = 2 * (256 + 256) * 144;
+            rc = finish(p.get(),
+                        gemmProgram(annot::MatrixOperand::BF16, false, annot::MatrixAccumulator::MFMA4, accumulate, 256,
+                                    256, 256, lds),
+                        flags);
+            if (rc == 0 && !(flags & GERN_PIPELINE_COMPILE_ONLY)) {
+                // The same program on data structures that promise whole tiles:
+                // eight wavefronts, no bounds tests.
+                gern_pipeline_s fast;
+                rc = finish(&fast,
+                            gemmProgram(annot::MatrixOperand::BF16, true, annot::MatrixAccumulator::MFMA8, accumulate,
+                                        256, 256, 512, lds),
+                            flags);
+                p->exact = std::move(fast.runner);
+            }
+        } else {
+            // gernels/mm.h, fma_lds_bytes()
+            const int64_t lds = 2 * 2 * 16 * 132 * 4;
+            rc = finish(p.get(),
+                        gemmProgram(annot::MatrixOperand::F32, false, annot::MatrixAccumulator::FMA, accumulate, 128, 128,
+                                    256, lds),
+                        flags);
+        }
         if (rc != 0) {
             return rc;
         }
@@ -322,9 +349,13 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 b{static_cast<float *>(const_cast<void *>(B)), K, N, N};
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
+    Runner *runner = p->runner.get();
+    if (p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0) {
+        runner = p->exact.get();
+    }
     try {
-        p->runner->setStream(stream);
-        p->runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
+        runner->setStream(stream);
+        runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
     } catch (const std::exception &e) {
         return fail(e.what());
     }

@@ -35,8 +35,9 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 
 // A window onto a row-major matrix in HBM: at most R x C, of which
-// rows x cols lie inside the matrix.
-template<int64_t R, int64_t C, typename T>
+// rows x cols lie inside the matrix.  EXACT promises that the window lies
+// wholly inside (rows == R, cols == C): gernels then skip every bounds test.
+template<int64_t R, int64_t C, typename T, bool EXACT>
 struct GlobalView {
     const T *data;
     int64_t lda;
@@ -45,9 +46,10 @@ struct GlobalView {
 };
 
 template<int64_t R, int64_t C>
-__device__ __forceinline__ GlobalView<R, C, float> MatrixF32::view(int64_t x, int64_t y) const {
+__device__ __forceinline__ GlobalView<R, C, float, false> MatrixF32::view(int64_t x, int64_t y) const {
     const int64_t r = row - x, c = col - y;
-    return GlobalView<R, C, float>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R, c < C ? (c < 0 ? 0 : c) : C};
+    return GlobalView<R, C, float, false>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
+                                          c < C ? (c < 0 ? 0 : c) : C};
 }
 
 // Row-major bf16 matrix in HBM (bit patterns).
@@ -58,25 +60,41 @@ struct MatrixBF16 {
     int64_t lda;
 
     template<int64_t R, int64_t C>
-    __device__ __forceinline__ GlobalView<R, C, uint16_t> view(int64_t x, int64_t y) const {
+    __device__ __forceinline__ GlobalView<R, C, uint16_t, false> view(int64_t x, int64_t y) const {
         const int64_t r = row - x, c = col - y;
-        return GlobalView<R, C, uint16_t>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
-                                          c < C ? (c < 0 ? 0 : c) : C};
+        return GlobalView<R, C, uint16_t, false>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
+                                                 c < C ? (c < 0 ? 0 : c) : C};
+    }
+    // For matrices whose extents are multiples of the window: the R x C
+    // window at (x, y), or what is left of the K extent when the window is
+    // deeper than the matrix (rows / cols then still say how much).
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ GlobalView<R, C, uint16_t, true> view_exact(int64_t x, int64_t y) const {
+        const int64_t r = row - x, c = col - y;
+        return GlobalView<R, C, uint16_t, true>{data + x * lda + y, lda, r < R ? r : R, c < C ? c : C};
     }
 };
 
 // ---------------------------------------------------------------------------
 // bf16 x bf16 -> fp32 on MFMA
 // ---------------------------------------------------------------------------
-// Accumulators of a BM x BN tile, spread over the 2 x 2 wavefronts of the
-// workgroup.  Wavefront (wm, wn) owns rows [wm*BM/2, ...) and columns
-// [wn*BN/2, ...); inside a 32 x 32 MFMA tile lane l, register i holds
-// row 8*(i/4) + 4*(l/32) + i%4, column l%32.
-template<int64_t BM, int64_t BN>
+// Accumulators of a BM x BN tile, spread over the NW wavefronts of the
+// workgroup, arranged 2 x (NW/2).  Wavefront (wm, wn) owns rows
+// [wm*BM/2, ...) and columns [wn*BN/(NW/2), ...); inside a 32 x 32 MFMA tile
+// lane l, register i holds row 8*(i/4) + 4*(l/32) + i%4, column l%32.
+//
+// NW = 8 (two wavefronts per SIMD) is the fast shape: one wavefront cannot
+// issue MFMAs back to back, two interleave and hide each other's LDS waits.
+template<int64_t BM, int64_t BN, int NW = 4>
 struct MfmaAcc {
-    static_assert(BM % 64 == 0 && BN % 64 == 0, "a wavefront owns whole 32 x 32 MFMA tiles");
-    static constexpr int TM = BM / 64;
-    static constexpr int TN = BN / 64;
+    static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
+    static constexpr int WC = NW / 2;           // wavefront columns
+    static constexpr int64_t WM = BM / 2;       // rows per wavefront
+    static constexpr int64_t WN = BN / WC;      // columns per wavefront
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "a wavefront owns whole 32 x 32 MFMA tiles");
+    static constexpr int TM = (int)(WM / 32);
+    static constexpr int TN = (int)(WN / 32);
+    static constexpr int threads = NW * kWaveSize;
     f32x16_t acc[TM][TN];
 
     __device__ __forceinline__ void destroy() {
@@ -89,19 +107,47 @@ __device__ __forceinline__ int wave_in_block() {
     return (int)(threadIdx.x / kWaveSize);
 }
 
-template<int64_t BM, int64_t BN, typename F>
-__device__ __forceinline__ void for_each_acc(F &&f) {
-    const int lane = lane_id();
-    const int w = wave_in_block();
-    const int64_t row0 = (int64_t)(w / 2) * (BM / 2) + 4 * (lane / 32);
-    const int64_t col0 = (int64_t)(w % 2) * (BN / 2) + (lane % 32);
+template<int64_t BM, int64_t BN, int NW>
+__device__ __forceinline__ MfmaAcc<BM, BN, NW> zero_acc() {
+    MfmaAcc<BM, BN, NW> t;
 #pragma unroll
-    for (int tm = 0; tm < MfmaAcc<BM, BN>::TM; tm++) {
+    for (int tm = 0; tm < MfmaAcc<BM, BN, NW>::TM; tm++) {
 #pragma unroll
-        for (int tn = 0; tn < MfmaAcc<BM, BN>::TN; tn++) {
+        for (int tn = 0; tn < MfmaAcc<BM, BN, NW>::TN; tn++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                f(tm, tn, i, row0 + tm * 32 + 8 * (i / 4) + (i % 4), col0 + tn * 32);
+                t.acc[tm][tn][i] = 0.f;
+            }
+        }
+    }
+    return t;
+}
+
+// ADD: C += tile (read-modify-write); otherwise C = tile.
+template<bool ADD, int64_t BM, int64_t BN, int NW>
+__device__ __forceinline__ void write_acc(const MatrixF32 &m, int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) {
+    using Acc = MfmaAcc<BM, BN, NW>;
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int64_t r0 = x + (int64_t)(w / Acc::WC) * Acc::WM + 4 * (lane / 32);
+    const int64_t c0 = y + (int64_t)(w % Acc::WC) * Acc::WN + (lane % 32);
+    const bool inside = (x + BM <= m.row) && (y + BN <= m.col);  // workgroup-uniform
+    const int ld = (int)m.lda;
+#pragma unroll
+    for (int tm = 0; tm < Acc::TM; tm++) {
+#pragma unroll
+        for (int tn = 0; tn < Acc::TN; tn++) {
+            float *p = m.data + (r0 + tm * 32) * m.lda + (c0 + tn * 32);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int dr = 8 * (i / 4) + (i % 4);
+                if (inside || ((r0 + tm * 32 + dr < m.row) && (c0 + tn * 32 < m.col))) {
+                    if (ADD) {
+                        p[dr * ld] += t.acc[tm][tn][i];
+                    } else {
+                        p[dr * ld] = t.acc[tm][tn][i];
+                    }
+                }
             }
         }
     }
@@ -109,28 +155,32 @@ __device__ __forceinline__ void for_each_acc(F &&f) {
 
 }  // namespace detail
 
-// C tile -> accumulators (C += A * B keeps what C held).
+// The accumulator tile is a DEFERRED update of C: it starts at zero and the
+// insert either adds it to what C holds (add_acc: C += A * B, the contract of
+// the reference's matrix_multiply) or overwrites C (store_acc: C = A * B,
+// which never reads C).  Loading C into the accumulators up front would give
+// the same sum, but parks up to 256 live values in VGPRs across the main loop.
 template<int64_t BM, int64_t BN>
-__device__ __forceinline__ MfmaAcc<BM, BN> MatrixF32::load_acc_mfma(int64_t x, int64_t y) const {
-    MfmaAcc<BM, BN> t;
-    detail::for_each_acc<BM, BN>([&](int tm, int tn, int i, int64_t r, int64_t c) {
-        const int64_t rr = x + r, cc = y + c;
-        t.acc[tm][tn][i] = (rr < row && cc < col) ? data[rr * lda + cc] : 0.f;
-    });
-    return t;
+__device__ __forceinline__ MfmaAcc<BM, BN, 4> MatrixF32::load_acc_mfma(int64_t, int64_t) const {
+    return detail::zero_acc<BM, BN, 4>();
 }
 
 template<int64_t BM, int64_t BN>
-__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN> &t) const {
-    detail::for_each_acc<BM, BN>([&](int tm, int tn, int i, int64_t r, int64_t c) {
-        const int64_t rr = x + r, cc = y + c;
-        if (rr < row && cc < col) {
-            data[rr * lda + cc] = t.acc[tm][tn][i];
-        }
-    });
+__device__ __forceinline__ MfmaAcc<BM, BN, 8> MatrixF32::load_acc_mfma8(int64_t, int64_t) const {
+    return detail::zero_acc<BM, BN, 8>();
 }
 
-constexpr int kMfmaBK = 64;                  // K depth of one LDS stage
+template<int64_t BM, int64_t BN, int NW>
+__device__ __forceinline__ void MatrixF32::add_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const {
+    detail::write_acc<true>(*this, x, y, t);
+}
+
+template<int64_t BM, int64_t BN, int NW>
+__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const {
+    detail::write_acc<false>(*this, x, y, t);
+}
+
+constexpr int kMfmaBK = 64;                      // K depth of one LDS stage
 constexpr int kMfmaRowBytes = 2 * kMfmaBK + 16;  // padded LDS row: 144 bytes
 
 // LDS needed by matrix_multiply on bf16 operands.
@@ -139,74 +189,92 @@ constexpr int64_t mfma_lds_bytes() {
     return 2 * (BM + BN) * kMfmaRowBytes;
 }
 
-template<int64_t BM, int64_t BN, int64_t KC>
-__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t> &A,
-                                                const GlobalView<KC, BN, uint16_t> &B, MfmaAcc<BM, BN> &C) {
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && BM <= 256 && BN <= 256, "tile shape");
-    constexpr int A_CHUNKS = BM * (kMfmaBK / 8) / 256;   // 16-byte chunks of A per thread per stage
-    constexpr int B_TASKS = (BN / 2) * (kMfmaBK / 8) / 256;  // 8-deep column pairs of B per thread per stage
-    static_assert(A_CHUNKS >= 1 && B_TASKS >= 1, "tile too small for 256 threads");
-    constexpr int STAGE_BYTES = (BM + BN) * kMfmaRowBytes;
+template<int64_t BM, int64_t BN, int64_t KC, int NW, bool EXACT>
+__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t, EXACT> &A,
+                                                const GlobalView<KC, BN, uint16_t, EXACT> &B, MfmaAcc<BM, BN, NW> &C) {
+    using Acc = MfmaAcc<BM, BN, NW>;
+    constexpr int T = Acc::threads;
+    static_assert(BM <= 256 && BN <= 256, "tile shape");
+    // Per stage, per thread: A_CHUNKS 16-byte pieces of A rows (8 bf16 along
+    // K), B_TASKS 8-deep column pairs of B.
+    constexpr int A_CHUNKS = (int)(BM * (kMfmaBK / 8) / T);
+    constexpr int B_TASKS = (int)((BN / 2) * (kMfmaBK / 8) / T);
+    static_assert(A_CHUNKS >= 1 && B_TASKS >= 1, "tile too small for the workgroup");
+    constexpr int A_ROW_STEP = T / (kMfmaBK / 8);  // rows between a thread's consecutive A chunks
+    constexpr int B_G_STEP = T / (int)(BN / 2);    // 8-deep K groups between a thread's consecutive B tasks
+    static_assert(B_G_STEP >= 1 && B_G_STEP * B_TASKS == kMfmaBK / 8, "B staging covers the stage exactly");
+    constexpr int STAGE_BYTES = (int)(BM + BN) * kMfmaRowBytes;
+    constexpr int TM = Acc::TM, TN = Acc::TN;
 
     const int tid = (int)threadIdx.x;
     const int lane = lane_id();
     const int w = detail::wave_in_block();
     const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
     const int nk = (int)((k_total + kMfmaBK - 1) / kMfmaBK);
+    if (nk == 0) {
+        return;
+    }
+    // EXACT windows: whole tiles, and a K extent that is a multiple of the
+    // stage depth; nothing needs a bounds test.
+
+    const int a_row = tid / (kMfmaBK / 8), a_kc = tid % (kMfmaBK / 8);
+    const int b_pair = tid % (int)(BN / 2), b_g = tid / (int)(BN / 2);
+    const uint16_t *a_ptr = A.data + (int64_t)a_row * A.lda + a_kc * 8;
+    const uint16_t *b_ptr = B.data + (int64_t)(8 * b_g) * B.lda + 2 * b_pair;
+    const int a_step = A_ROW_STEP * (int)A.lda;    // elements between chunks
+    const int b_step = 8 * B_G_STEP * (int)B.lda;  // elements between tasks
+    const int b_ld = (int)B.lda;
 
     uint4 ra[A_CHUNKS];
     uint32_t rb[B_TASKS][8];
 
     auto fetch = [&](int kt) {
         const int64_t k0 = (int64_t)kt * kMfmaBK;
+        if constexpr (EXACT) {
 #pragma unroll
-        for (int j = 0; j < A_CHUNKS; j++) {
-            const int c = tid + 256 * j;
-            const int64_t r = c / 8, kk = k0 + (c % 8) * 8;
-            uint4 v = make_uint4(0u, 0u, 0u, 0u);
-            if (r < A.rows && kk + 7 < k_total) {
-                v = *reinterpret_cast<const uint4 *>(A.data + r * A.lda + kk);
-            } else if (r < A.rows && kk < k_total) {
-                uint16_t e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                for (int q = 0; q < 8; q++) {
-                    if (kk + q < k_total) e[q] = A.data[r * A.lda + kk + q];
-                }
-                v = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+            for (int j = 0; j < A_CHUNKS; j++) {
+                ra[j] = *reinterpret_cast<const uint4 *>(a_ptr + k0 + j * a_step);
             }
-            ra[j] = v;
-        }
+            const uint16_t *bp = b_ptr + k0 * B.lda;
 #pragma unroll
-        for (int j = 0; j < B_TASKS; j++) {
-            const int id = tid + 256 * j;
-            const int64_t n = 2 * (id % (BN / 2)), kk = k0 + 8 * (id / (BN / 2));
+            for (int j = 0; j < B_TASKS; j++) {
 #pragma unroll
-            for (int q = 0; q < 8; q++) {
-                uint32_t v = 0u;
-                if (kk + q < k_total) {
-                    const uint16_t *p = B.data + (kk + q) * B.lda + n;
-                    if (n + 1 < B.cols) {
-                        v = *reinterpret_cast<const uint32_t *>(p);
-                    } else if (n < B.cols) {
-                        v = p[0];
-                    }
+                for (int q = 0; q < 8; q++) {
+                    rb[j][q] = *reinterpret_cast<const uint32_t *>(bp + j * b_step + q * b_ld);
                 }
-                rb[j][q] = v;
+            }
+        } else {
+            // Ragged tile: the same accesses, each under a predicate.  A row
+            // of A is read in whole 16-byte pieces and a row of B in whole
+            // column pairs (the caller guarantees K % 8 == 0 and N % 2 == 0).
+#pragma unroll
+            for (int j = 0; j < A_CHUNKS; j++) {
+                const bool ok = (a_row + j * A_ROW_STEP < A.rows) && (k0 + a_kc * 8 < k_total);
+                ra[j] = ok ? *reinterpret_cast<const uint4 *>(a_ptr + k0 + j * a_step) : make_uint4(0u, 0u, 0u, 0u);
+            }
+            const uint16_t *bp = b_ptr + k0 * B.lda;
+            const bool col_ok = 2 * b_pair < B.cols;
+#pragma unroll
+            for (int j = 0; j < B_TASKS; j++) {
+                const int64_t kk = k0 + 8 * (b_g + j * B_G_STEP);
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const bool ok = col_ok && (kk + q < k_total);
+                    rb[j][q] = ok ? *reinterpret_cast<const uint32_t *>(bp + j * b_step + q * b_ld) : 0u;
+                }
             }
         }
     };
 
     auto stash = [&](int buf) {
-        unsigned char *a_lds = gern_lds + buf * STAGE_BYTES;
-        unsigned char *b_lds = a_lds + BM * kMfmaRowBytes;
+        unsigned char *a_lds = gern_lds + buf * STAGE_BYTES + a_row * kMfmaRowBytes + a_kc * 16;
+        unsigned char *b_lds = gern_lds + buf * STAGE_BYTES + (int)BM * kMfmaRowBytes + (2 * b_pair) * kMfmaRowBytes + b_g * 16;
 #pragma unroll
         for (int j = 0; j < A_CHUNKS; j++) {
-            const int c = tid + 256 * j;
-            *reinterpret_cast<uint4 *>(a_lds + (c / 8) * kMfmaRowBytes + (c % 8) * 16) = ra[j];
+            *reinterpret_cast<uint4 *>(a_lds + j * A_ROW_STEP * kMfmaRowBytes) = ra[j];
         }
 #pragma unroll
         for (int j = 0; j < B_TASKS; j++) {
-            const int id = tid + 256 * j;
-            const int n = 2 * (id % (BN / 2)), g = id / (BN / 2);
             // rb[j][q] = {B[k+q][n] (low half), B[k+q][n+1] (high half)}: split
             // into the K-contiguous vectors of column n and column n+1.
             uint4 lo, hi;
@@ -218,44 +286,94 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
             hi.y = __builtin_amdgcn_perm(rb[j][3], rb[j][2], 0x07060302u);
             hi.z = __builtin_amdgcn_perm(rb[j][5], rb[j][4], 0x07060302u);
             hi.w = __builtin_amdgcn_perm(rb[j][7], rb[j][6], 0x07060302u);
-            *reinterpret_cast<uint4 *>(b_lds + n * kMfmaRowBytes + g * 16) = lo;
-            *reinterpret_cast<uint4 *>(b_lds + (n + 1) * kMfmaRowBytes + g * 16) = hi;
+            // Column n goes to LDS row n, column n+1 to row n+1.  Eight
+            // consecutive lanes must hit eight different 16-byte bank groups;
+            // rows 2p (p = 0..7) only reach four, so lanes with bit 2 of p set
+            // write their odd row first: rows 0,2,4,6,9,11,13,15.
+            const bool odd_first = (b_pair & 4) != 0;
+            *reinterpret_cast<uint4 *>(b_lds + (odd_first ? kMfmaRowBytes : 0) + j * B_G_STEP * 16) = odd_first ? hi : lo;
+            *reinterpret_cast<uint4 *>(b_lds + (odd_first ? 0 : kMfmaRowBytes) + j * B_G_STEP * 16) = odd_first ? lo : hi;
         }
     };
 
-    if (nk == 0) {
-        return;
-    }
-    fetch(0);
+    // Workgroups that run at the same time start their walk over K at
+    // different steps (and wrap around).  With a power-of-two row pitch the
+    // rows of one K step all fall into the same memory channel; if every
+    // workgroup asked for the same step at once, one channel would serve the
+    // whole chip.  The sum over K does not depend on where the walk starts.
+    const int k_shift = (int)((blockIdx.x + gridDim.x * blockIdx.y) % (unsigned)nk);
+    auto step_of = [&](int kt) {
+        const int s = kt + k_shift;
+        return s >= nk ? s - nk : s;
+    };
+
+    fetch(step_of(0));
     stash(0);
     __syncthreads();
 
-    const int a_row0 = (w / 2) * (int)(BM / 2) + (lane % 32);
-    const int b_row0 = (w % 2) * (int)(BN / 2) + (lane % 32);
-    const int k_off = (lane / 32) * 16;
+    // This lane's fragment addresses inside a stage: row (lane % 32) of each
+    // 32-row MFMA tile, 16 bytes at K offset 8 * (lane / 32) of each K step.
+    const int a_frag = ((w / Acc::WC) * (int)Acc::WM + (lane % 32)) * kMfmaRowBytes + (lane / 32) * 16;
+    const int b_frag = (int)BM * kMfmaRowBytes + ((w % Acc::WC) * (int)Acc::WN + (lane % 32)) * kMfmaRowBytes + (lane / 32) * 16;
 
     for (int kt = 0; kt < nk; kt++) {
         if (kt + 1 < nk) {
-            fetch(kt + 1);
+            fetch(step_of(kt + 1));
         }
-        const unsigned char *a_lds = gern_lds + (kt & 1) * STAGE_BYTES;
-        const unsigned char *b_lds = a_lds + BM * kMfmaRowBytes;
+        const unsigned char *stage = gern_lds + (kt & 1) * STAGE_BYTES;
+        if constexpr (NW == 4) {
+            // One wavefront per SIMD: read the next K step's fragments while
+            // this step's MFMAs run.
+            bf16x8_t af[2][TM], bfr[2][TN];
 #pragma unroll
-        for (int s = 0; s < kMfmaBK / 16; s++) {
-            bf16x8_t af[MfmaAcc<BM, BN>::TM], bfr[MfmaAcc<BM, BN>::TN];
-#pragma unroll
-            for (int tm = 0; tm < MfmaAcc<BM, BN>::TM; tm++) {
-                af[tm] = *reinterpret_cast<const bf16x8_t *>(a_lds + (a_row0 + tm * 32) * kMfmaRowBytes + s * 32 + k_off);
+            for (int tm = 0; tm < TM; tm++) {
+                af[0][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes);
             }
 #pragma unroll
-            for (int tn = 0; tn < MfmaAcc<BM, BN>::TN; tn++) {
-                bfr[tn] = *reinterpret_cast<const bf16x8_t *>(b_lds + (b_row0 + tn * 32) * kMfmaRowBytes + s * 32 + k_off);
+            for (int tn = 0; tn < TN; tn++) {
+                bfr[0][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_frag + tn * 32 * kMfmaRowBytes);
             }
 #pragma unroll
-            for (int tm = 0; tm < MfmaAcc<BM, BN>::TM; tm++) {
+            for (int s = 0; s < kMfmaBK / 16; s++) {
+                const int cur = s & 1, nxt = cur ^ 1;
+                if (s + 1 < kMfmaBK / 16) {
 #pragma unroll
-                for (int tn = 0; tn < MfmaAcc<BM, BN>::TN; tn++) {
-                    C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[tm], bfr[tn], C.acc[tm][tn], 0, 0, 0);
+                    for (int tm = 0; tm < TM; tm++) {
+                        af[nxt][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + (s + 1) * 32);
+                    }
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        bfr[nxt][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_frag + tn * 32 * kMfmaRowBytes + (s + 1) * 32);
+                    }
+                }
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][tm], bfr[cur][tn], C.acc[tm][tn], 0, 0, 0);
+                    }
+                }
+            }
+        } else {
+            // Two wavefronts per SIMD cover each other's LDS waits; single
+            // fragment buffers keep each within half the register file.
+#pragma unroll
+            for (int s = 0; s < kMfmaBK / 16; s++) {
+                bf16x8_t af[TM], bfr[TN];
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+                    af[tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + s * 32);
+                }
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    bfr[tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_frag + tn * 32 * kMfmaRowBytes + s * 32);
+                }
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[tm], bfr[tn], C.acc[tm][tn], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -296,40 +414,55 @@ __device__ __forceinline__ void for_each_fma_acc(F &&f) {
 
 }  // namespace detail
 
+// Like the MFMA tile, a deferred update of C: zero at query, added to
+// (add_acc) or written over (store_acc) C at insert.
 template<int64_t BM, int64_t BN>
-__device__ __forceinline__ FmaAcc<BM, BN> MatrixF32::load_acc_fma(int64_t x, int64_t y) const {
+__device__ __forceinline__ FmaAcc<BM, BN> MatrixF32::load_acc_fma(int64_t, int64_t) const {
     FmaAcc<BM, BN> t;
-    detail::for_each_fma_acc([&](int i, int j, int64_t r, int64_t c) {
-        const int64_t rr = x + r, cc = y + c;
-        const float *p = data + rr * lda + cc;
-        if (rr < row && cc + 3 < col && ((((uint64_t)p) & 15u) == 0)) {
-            const float4 v = *reinterpret_cast<const float4 *>(p);
-            t.acc[i][j] = v.x;
-            t.acc[i][j + 1] = v.y;
-            t.acc[i][j + 2] = v.z;
-            t.acc[i][j + 3] = v.w;
-        } else {
-            for (int e = 0; e < 4; e++) {
-                t.acc[i][j + e] = (rr < row && cc + e < col) ? p[e] : 0.f;
-            }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            t.acc[i][j] = 0.f;
         }
-    });
+    }
     return t;
 }
 
-template<int64_t BM, int64_t BN>
-__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const {
-    detail::for_each_fma_acc([&](int i, int j, int64_t r, int64_t c) {
+namespace detail {
+
+template<bool ADD, int64_t BM, int64_t BN>
+__device__ __forceinline__ void write_fma_acc(const MatrixF32 &m, int64_t x, int64_t y, const FmaAcc<BM, BN> &t) {
+    for_each_fma_acc([&](int i, int j, int64_t r, int64_t c) {
         const int64_t rr = x + r, cc = y + c;
-        float *p = data + rr * lda + cc;
-        if (rr < row && cc + 3 < col && ((((uint64_t)p) & 15u) == 0)) {
-            *reinterpret_cast<float4 *>(p) = make_float4(t.acc[i][j], t.acc[i][j + 1], t.acc[i][j + 2], t.acc[i][j + 3]);
+        float *p = m.data + rr * m.lda + cc;
+        if (rr < m.row && cc + 3 < m.col && ((((uint64_t)p) & 15u) == 0)) {
+            float4 v = make_float4(t.acc[i][j], t.acc[i][j + 1], t.acc[i][j + 2], t.acc[i][j + 3]);
+            if (ADD) {
+                const float4 o = *reinterpret_cast<const float4 *>(p);
+                v = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+            }
+            *reinterpret_cast<float4 *>(p) = v;
         } else {
             for (int e = 0; e < 4; e++) {
-                if (rr < row && cc + e < col) p[e] = t.acc[i][j + e];
+                if (rr < m.row && cc + e < m.col) {
+                    p[e] = ADD ? p[e] + t.acc[i][j + e] : t.acc[i][j + e];
+                }
             }
         }
     });
+}
+
+}  // namespace detail
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const {
+    detail::write_fma_acc<false>(*this, x, y, t);
+}
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::add_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const {
+    detail::write_fma_acc<true>(*this, x, y, t);
 }
 
 constexpr int kFmaBK = 16;
@@ -341,8 +474,8 @@ constexpr int64_t fma_lds_bytes() {
 }
 
 template<int64_t BM, int64_t BN, int64_t KC>
-__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float> &A, const GlobalView<KC, BN, float> &B,
-                                                FmaAcc<BM, BN> &C) {
+__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float, false> &A,
+                                                const GlobalView<KC, BN, float, false> &B, FmaAcc<BM, BN> &C) {
     constexpr int STAGE_FLOATS = 2 * kFmaBK * kFmaLd;
     float *lds = reinterpret_cast<float *>(gern_lds);
     const int tid = (int)threadIdx.x;
@@ -410,12 +543,20 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float> 
     if (nk == 0) {
         return;
     }
-    fetch(0);
+    // Concurrent workgroups start their walk over K at different steps, so
+    // that they do not all pull on the same memory channel (see the MFMA
+    // gernel above).
+    const int k_shift = (int)((blockIdx.x + gridDim.x * blockIdx.y) % (unsigned)nk);
+    auto step_of = [&](int kt) {
+        const int s = kt + k_shift;
+        return s >= nk ? s - nk : s;
+    };
+    fetch(step_of(0));
     stash(0);
     __syncthreads();
     for (int kt = 0; kt < nk; kt++) {
         if (kt + 1 < nk) {
-            fetch(kt + 1);
+            fetch(step_of(kt + 1));
         }
         const float *a_lds = lds + (kt & 1) * STAGE_FLOATS;
         const float *b_lds = a_lds + kFmaBK * kFmaLd;

@@ -98,7 +98,7 @@ __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y,
 // S = scale * Q K^T for the 16 rows of Q in view; columns past the last key
 // get -inf so that they vanish from the softmax.
 template<int64_t R, int64_t N, int64_t D>
-__device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t> &Q, const GlobalView<N, D, uint16_t> &K,
+__device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false> &Q, const GlobalView<N, D, uint16_t, false> &K,
                                           RowBlock<R, N> &S, float scale) {
     static_assert(D % 32 == 0 && D <= 256, "head dimension in MFMA K steps of 32");
     constexpr int KS = (int)(D / 32);

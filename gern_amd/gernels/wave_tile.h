@@ -52,9 +52,9 @@ __device__ __forceinline__ WaveVec<R> allocate_wave_vec() {
 
 // Defined in gernels/mm.h: a window onto a matrix in HBM (no data movement) and
 // the two block-distributed accumulator tiles of the GEMM gernels.
-template<int64_t R, int64_t C, typename T>
+template<int64_t R, int64_t C, typename T, bool EXACT>
 struct GlobalView;
-template<int64_t BM, int64_t BN>
+template<int64_t BM, int64_t BN, int NW>
 struct MfmaAcc;
 template<int64_t BM, int64_t BN>
 struct FmaAcc;
@@ -73,15 +73,21 @@ struct MatrixF32 {
 
     // GEMM operand / result access (gernels/mm.h).
     template<int64_t R, int64_t C>
-    __device__ __forceinline__ GlobalView<R, C, float> view(int64_t x, int64_t y) const;
+    __device__ __forceinline__ GlobalView<R, C, float, false> view(int64_t x, int64_t y) const;
     template<int64_t BM, int64_t BN>
-    __device__ __forceinline__ MfmaAcc<BM, BN> load_acc_mfma(int64_t x, int64_t y) const;
+    __device__ __forceinline__ MfmaAcc<BM, BN, 4> load_acc_mfma(int64_t x, int64_t y) const;
     template<int64_t BM, int64_t BN>
-    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN> &t) const;
+    __device__ __forceinline__ MfmaAcc<BM, BN, 8> load_acc_mfma8(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN, int NW>
+    __device__ __forceinline__ void add_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const;
+    template<int64_t BM, int64_t BN, int NW>
+    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const;
     template<int64_t BM, int64_t BN>
     __device__ __forceinline__ FmaAcc<BM, BN> load_acc_fma(int64_t x, int64_t y) const;
     template<int64_t BM, int64_t BN>
     __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void add_acc(int64_t x, int64_t y, const FmaAcc<BM, BN> &t) const;
     // Fused QK^T -> softmax result access (gernels/qk_softmax.h).
     template<int64_t R, int64_t N>
     __device__ __forceinline__ RowBlock<R, N> view_row_block(int64_t x, int64_t y) const;

@@ -30,7 +30,9 @@ enum {
      * GPU and cannot be run. */
     GERN_PIPELINE_COMPILE_ONLY = 1,
     /* Launch workgroups in plain blockIdx order (no XCD-aware renumbering). */
-    GERN_PIPELINE_NO_XCD_REMAP = 2
+    GERN_PIPELINE_NO_XCD_REMAP = 2,
+    /* GEMM only: C = A * B (C is written, never read) instead of C += A * B. */
+    GERN_PIPELINE_GEMM_OVERWRITE = 4
 };
 
 /* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
@@ -57,9 +59,12 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
 int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows, int64_t ld,
                      void *stream);
 
-/* Dense GEMM C += A * B, row-major, A is M x K, B is K x N, C is M x N fp32.
+/* Dense GEMM C += A * B (or C = A * B with GERN_PIPELINE_GEMM_OVERWRITE),
+ * row-major, A is M x K, B is K x N, C is M x N fp32.
  * variant 0: fp32 inputs, vector-ALU FMAs.
- * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA.
+ * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA; needs
+ *            K % 8 == 0 and N % 2 == 0.  Shapes with M % 256 == N % 256 ==
+ *            K % 64 == 0 take a kernel without bounds tests.
  * Composes Tile(i)(Tile(j)(Reduce(k)(matrix_multiply))) as
  * gernels/mm/kernel_3.cu:61-75 does. */
 int gern_gemm_create(int variant, int flags, gern_pipeline *out);
