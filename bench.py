@@ -51,6 +51,44 @@ def time_launches(fn, warmup, steps, torch, gern_amd):
     return wall, start.elapsed_ms_until(stop) / steps
 
 
+COPY_SRC = r"""
+extern "C" __global__ void __launch_bounds__(256) gern_copy_f4(const float4 *in, float4 *out, long long n)
+{
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = in[i];
+}
+"""
+
+
+def copy_calibration(torch, gern_amd, warmup, steps):
+    """A plain float4 copy of 256 MiB through the same C ABI: the HBM rate a
+    trivial kernel reaches on this device, and the kernel of known size that
+    the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    import ctypes as C
+    hip = gern_amd.hip_lib()
+    mod, ker = C.c_void_p(), C.c_void_p()
+    names = (C.c_char_p * 1)(b"gern_copy_f4")
+    if hip.gern_hip_compile(COPY_SRC.encode(), names, 1, None, 0, None, C.byref(mod)) != 0 or \
+       hip.gern_hip_get_kernel(mod, b"gern_copy_f4", C.byref(ker)) != 0:
+        raise gern_amd.GernError(gern_amd._hip_error())
+    nbytes = 256 << 20
+    src = torch.ones(nbytes // 4, device="cuda")
+    dst = torch.zeros_like(src)
+    n = C.c_longlong(nbytes // 16)
+    a, b = C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())
+    params = (C.c_void_p * 3)(C.cast(C.byref(a), C.c_void_p), C.cast(C.byref(b), C.c_void_p), C.cast(C.byref(n), C.c_void_p))
+    grid = (C.c_uint32 * 3)((nbytes // 16 + 255) // 256, 1, 1)
+    block = (C.c_uint32 * 3)(256, 1, 1)
+
+    def launch():
+        if hip.gern_hip_launch(ker, grid, block, 0, params, None) != 0:
+            raise gern_amd.GernError(gern_amd._hip_error())
+    wall, ev = time_launches(launch, warmup, steps, torch, gern_amd)
+    assert bool((dst == 1).all())
+    return {"GB/s": 2 * nbytes / (ev * 1e-3) / 1e9, "ms": ev, "frac_hbm": 2 * nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "kernel": "gern_copy_f4", "bytes_read": nbytes, "bytes_written": nbytes}
+
+
 def cpu_baseline_blur(img_np):
     """The same composed pipeline on ONE host core."""
     from oracle import oracle as o
@@ -91,7 +129,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only this workload (blur, softmax, gemm_f32, gemm_bf16, qk_softmax)")
+    ap.add_argument("--only", default="", help="run only this workload (blur, softmax, gemm_f32, gemm_bf16, qk_softmax, copy)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -201,6 +239,11 @@ def main():
         workloads["qk_softmax_4096x4096x128"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "TFLOP/s": tf,
                                                  "frac_mfma": tf / MFMA_BF16_PEAK_TFLOPS, "kernel": qk.kernel_name}
         log("qk softmax 4096x4096x128: %.1f us  %.0f GB/s (%.1f%% HBM)  %.1f TFLOP/s" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS, tf))
+
+    # ---- calibration: plain copy of known size ------------------------------
+    if want("copy"):
+        workloads["copy_256MiB"] = copy_calibration(torch, gern_amd, args.warmup, steps2)
+        log("copy 256 MiB: %.1f us  %.0f GB/s" % (workloads["copy_256MiB"]["ms"] * 1e3, workloads["copy_256MiB"]["GB/s"]))
 
     if result is None:
         result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "", "n_gpus": 1,

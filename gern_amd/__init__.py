@@ -66,6 +66,11 @@ def _load():
     if hasattr(pipes, "gern_qk_softmax_create"):
         pipes.gern_qk_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
         pipes.gern_qk_softmax_run.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
+    cpp = C.POINTER(C.c_char_p)
+    hip.gern_hip_compile.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(vp)]
+    hip.gern_hip_compile_only.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(sz)]
+    hip.gern_hip_get_kernel.argtypes = [vp, C.c_char_p, C.POINTER(vp)]
+    hip.gern_hip_launch.argtypes = [vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(vp), vp]
     hip.gern_hip_event_create.argtypes = [C.POINTER(vp)]
     hip.gern_hip_event_record.argtypes = [vp, vp]
     hip.gern_hip_event_elapsed_ms.argtypes = [vp, vp, C.POINTER(C.c_float)]

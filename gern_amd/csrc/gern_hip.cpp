@@ -6,7 +6,9 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -149,6 +151,21 @@ int compile_program(const char *source, const char *const *name_exprs, int n_nam
     out.code.resize(code_size);
     hiprtcGetCode(prog, out.code.data());
     hiprtcDestroyProgram(&prog);
+    // Like the reference Runner, which leaves its generated source and shared
+    // object in `prefix` (src/codegen/runner.cpp:20-35): with GERN_HIP_KEEP_DIR
+    // set, the source and the code object are kept there for inspection.
+    if (const char *dir = std::getenv("GERN_HIP_KEEP_DIR")) {
+        static std::atomic<int> serial{0};
+        const std::string base = std::string(dir) + "/gern_generated_" + std::to_string(serial++);
+        if (FILE *f = std::fopen((base + ".hip").c_str(), "w")) {
+            std::fputs(source, f);
+            std::fclose(f);
+        }
+        if (FILE *f = std::fopen((base + ".hsaco").c_str(), "wb")) {
+            std::fwrite(out.code.data(), 1, out.code.size(), f);
+            std::fclose(f);
+        }
+    }
     return GERN_HIP_OK;
 }
 

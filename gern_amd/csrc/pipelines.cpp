@@ -52,6 +52,8 @@ struct gern_pipeline_s {
     std::unique_ptr<Runner> exact;   // GEMM bf16: the kernel for shapes that are multiples of the tile
     std::string source;
     std::string kernel_name;
+    std::string exact_source, exact_kernel_name;
+    bool last_run_exact = false;
     // blur
     int64_t nx = 0, ny = 0, stride = 0;
     // softmax / qk
@@ -301,7 +303,7 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                         gemmProgram(annot::MatrixOperand::BF16, false, annot::MatrixAccumulator::MFMA4, accumulate, 256,
                                     256, 256, lds),
                         flags);
-            if (rc == 0 && !(flags & GERN_PIPELINE_COMPILE_ONLY)) {
+            if (rc == 0) {
                 // The same program on data structures that promise whole tiles:
                 // eight wavefronts, no bounds tests.
                 gern_pipeline_s fast;
@@ -310,6 +312,10 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                                         256, 256, 512, lds),
                             flags);
                 p->exact = std::move(fast.runner);
+                p->exact_source = fast.source;
+                p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
+                // The shape the pipeline is built for is the exact one.
+                p->last_run_exact = true;
             }
         } else {
             // gernels/mm.h, fma_lds_bytes()
@@ -350,7 +356,8 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    if (p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0) {
+    p->last_run_exact = p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;
+    if (p->last_run_exact) {
         runner = p->exact.get();
     }
     try {
@@ -435,7 +442,10 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
 }
 
 const char *gern_pipeline_source(gern_pipeline p) {
-    return p ? p->source.c_str() : "";
+    if (p == nullptr) {
+        return "";
+    }
+    return p->last_run_exact && !p->exact_source.empty() ? p->exact_source.c_str() : p->source.c_str();
 }
 
 const char *gern_pipeline_kernel_name(gern_pipeline p) {
@@ -444,6 +454,9 @@ const char *gern_pipeline_kernel_name(gern_pipeline p) {
     }
     if (p->kernel_name.empty() && p->runner) {
         p->kernel_name = p->runner->getKernelName();
+    }
+    if (p->last_run_exact && !p->exact_kernel_name.empty()) {
+        return p->exact_kernel_name.c_str();
     }
     return p->kernel_name.c_str();
 }

@@ -30,6 +30,7 @@ namespace gernels {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // Dynamic LDS of the kernel; the launch sizes it (Global(..., smem_size)).
 extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
@@ -225,7 +226,9 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
     const int b_step = 8 * B_G_STEP * (int)B.lda;  // elements between tasks
     const int b_ld = (int)B.lda;
 
-    uint4 ra[A_CHUNKS];
+    // Native vector types: selecting between two of HIP's uint4 structs
+    // (cond ? a : b) takes their addresses and sends both to scratch memory.
+    u32x4_t ra[A_CHUNKS];
     uint32_t rb[B_TASKS][8];
 
     auto fetch = [&](int kt) {
@@ -233,7 +236,7 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
         if constexpr (EXACT) {
 #pragma unroll
             for (int j = 0; j < A_CHUNKS; j++) {
-                ra[j] = *reinterpret_cast<const uint4 *>(a_ptr + k0 + j * a_step);
+                ra[j] = *reinterpret_cast<const u32x4_t *>(a_ptr + k0 + j * a_step);
             }
             const uint16_t *bp = b_ptr + k0 * B.lda;
 #pragma unroll
@@ -250,7 +253,10 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
 #pragma unroll
             for (int j = 0; j < A_CHUNKS; j++) {
                 const bool ok = (a_row + j * A_ROW_STEP < A.rows) && (k0 + a_kc * 8 < k_total);
-                ra[j] = ok ? *reinterpret_cast<const uint4 *>(a_ptr + k0 + j * a_step) : make_uint4(0u, 0u, 0u, 0u);
+                ra[j] = u32x4_t{0u, 0u, 0u, 0u};
+                if (ok) {
+                    ra[j] = *reinterpret_cast<const u32x4_t *>(a_ptr + k0 + j * a_step);
+                }
             }
             const uint16_t *bp = b_ptr + k0 * B.lda;
             const bool col_ok = 2 * b_pair < B.cols;
@@ -271,13 +277,13 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
         unsigned char *b_lds = gern_lds + buf * STAGE_BYTES + (int)BM * kMfmaRowBytes + (2 * b_pair) * kMfmaRowBytes + b_g * 16;
 #pragma unroll
         for (int j = 0; j < A_CHUNKS; j++) {
-            *reinterpret_cast<uint4 *>(a_lds + j * A_ROW_STEP * kMfmaRowBytes) = ra[j];
+            *reinterpret_cast<u32x4_t *>(a_lds + j * A_ROW_STEP * kMfmaRowBytes) = ra[j];
         }
 #pragma unroll
         for (int j = 0; j < B_TASKS; j++) {
             // rb[j][q] = {B[k+q][n] (low half), B[k+q][n+1] (high half)}: split
             // into the K-contiguous vectors of column n and column n+1.
-            uint4 lo, hi;
+            u32x4_t lo, hi;
             lo.x = __builtin_amdgcn_perm(rb[j][1], rb[j][0], 0x05040100u);
             lo.y = __builtin_amdgcn_perm(rb[j][3], rb[j][2], 0x05040100u);
             lo.z = __builtin_amdgcn_perm(rb[j][5], rb[j][4], 0x05040100u);
@@ -291,8 +297,8 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
             // rows 2p (p = 0..7) only reach four, so lanes with bit 2 of p set
             // write their odd row first: rows 0,2,4,6,9,11,13,15.
             const bool odd_first = (b_pair & 4) != 0;
-            *reinterpret_cast<uint4 *>(b_lds + (odd_first ? kMfmaRowBytes : 0) + j * B_G_STEP * 16) = odd_first ? hi : lo;
-            *reinterpret_cast<uint4 *>(b_lds + (odd_first ? 0 : kMfmaRowBytes) + j * B_G_STEP * 16) = odd_first ? lo : hi;
+            *reinterpret_cast<u32x4_t *>(b_lds + (odd_first ? kMfmaRowBytes : 0) + j * B_G_STEP * 16) = odd_first ? hi : lo;
+            *reinterpret_cast<u32x4_t *>(b_lds + (odd_first ? 0 : kMfmaRowBytes) + j * B_G_STEP * 16) = odd_first ? lo : hi;
         }
     };
 

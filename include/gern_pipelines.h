@@ -81,7 +81,9 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
 int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M,
                         int64_t N, float scale, void *stream);
 
-/* The generated device source (owned by the pipeline, valid until destroy). */
+/* The generated device source (owned by the pipeline, valid until destroy).
+ * A pipeline that holds more than one kernel (bf16 GEMM) reports the one its
+ * last run used; before any run, the one for whole-tile shapes. */
 const char *gern_pipeline_source(gern_pipeline p);
 /* The name expression of the instantiated kernel, e.g. "function_7<252, 8, 3>". */
 const char *gern_pipeline_kernel_name(gern_pipeline p);
