@@ -29,6 +29,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA
 FP32_VECTOR_PEAK_TFLOPS = 157.3
+# HBM bytes one launch of the headline kernel moves, from the FETCH_SIZE and
+# WRITE_SIZE counters scaled by the plain-copy calibration kernel below
+# (profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from
+# inside this process; the figure is re-measured whenever the kernel changes.
+BLUR_XYX_8192_TRAFFIC_BYTES = 539309230
 
 
 def log(*a):
@@ -160,7 +165,7 @@ def main():
         nbytes = img.nbytes + d_out.numel() * 4
         gbs = nbytes / (wall * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": nbytes / (ev * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                "frac": nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": BLUR_XYX_8192_TRAFFIC_BYTES,
                 "kernel": blur.kernel_name, "kernel_ms": ev, "algorithmic_bytes": nbytes}
         workloads["blur_xyx_8192"] = {"GB/s": gbs, "ms": wall, "frac_hbm": gbs / HBM_PEAK_GBS}
         log("blur xyx 8192^2: %.1f us/launch  %.0f GB/s  (%.1f%% of HBM peak)" % (wall * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
