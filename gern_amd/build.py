@@ -48,9 +48,22 @@ def build_gernel_check():
     run([os.path.join(ROCM, "bin", "hipcc")] + HIPFLAGS + ["-c", "--cuda-device-only", src, "-o", out])
 
 
+def build_cpp_tests():
+    """The C++ front-end / lowering test programs (tests/cpp/*.cpp -> tests/cpp/bin/)."""
+    tdir = os.path.join(ROOT, "tests", "cpp")
+    bindir = os.path.join(tdir, "bin")
+    os.makedirs(bindir, exist_ok=True)
+    rpath = "-Wl,-rpath,$ORIGIN/../../../gern_amd:" + os.path.join(ROCM, "lib")
+    for src in sorted(glob.glob(os.path.join(tdir, "test_*.cpp"))):
+        exe = os.path.join(bindir, os.path.splitext(os.path.basename(src))[0])
+        run(["g++", "-std=c++20", "-O1", "-I" + tdir] + [f for f in CXXFLAGS if f.startswith("-I") or f.startswith("-D")] +
+            [src, "-L" + HERE, "-lgern", "-lgern_hip", rpath, "-o", exe])
+
+
 def build_all():
     build_native()
     build_gernel_check()
+    build_cpp_tests()
 
 
 if __name__ == "__main__":

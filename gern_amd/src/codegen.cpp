@@ -239,6 +239,17 @@ public:
         if (!f.template_args.empty()) {
             os << "<";
             for (size_t i = 0; i < f.template_args.size(); i++) {
+                // A template argument is a compile-time value: every variable
+                // in it must have been bound (reference: the same complaint is
+                // raised for the generated function's own template
+                // parameters, src/codegen/codegen.cpp:179-183).
+                const Argument &targ = f.template_args[i];
+                for (const auto &v : targ.isExpr() ? getVariables(targ.getExpr()) : std::set<Variable>{}) {
+                    if (!v.isConstExpr()) {
+                        throw error::UserError(v.getName() + " must be bound to an int64_t, it is a template argument of " +
+                                               f.name);
+                    }
+                }
                 os << (i ? ", " : "") << gen(f.template_args[i]);
             }
             os << ">";
@@ -550,7 +561,10 @@ std::string CodeGenerator::generate_code(Composable c) {
     for (size_t i = 0; i < parameters.size(); i++) {
         const Parameter &p = parameters[i];
         std::string name = p.isData() ? p.getADTPtr().getName() : p.getVar().getName();
-        out << (i ? ", " : "") << p.getType() << (device ? " " : " &") << name;
+        // Host functions take data structures by reference (the callee's
+        // insert must reach the caller's object); variables go by value, so
+        // that a caller may pass a compile-time constant.
+        out << (i ? ", " : "") << p.getType() << ((device || !p.isData()) ? " " : " &") << name;
     }
     out << ") {\n";
     if (device && em.uses_block_units && options.xcd_remap) {

@@ -1,0 +1,396 @@
+// Lowering to ONE HIP kernel for gfx950 and running it: unmapped loops,
+// loops mapped to blocks / threads / wavefronts, repeated units, explicit
+// launch dimensions, dynamic LDS with an allocator, LDS-staged tiles.
+//
+// The cases follow the reference's device lowering tests: test/test-gpu-array.cu,
+// test-set-grid.cu, test-dynamic-shared.cu, test-gpu-matrix.cu.
+//
+// With GERN_TEST_COMPILE_ONLY=1 every program is generated and compiled for
+// gfx950 with hiprtc but not loaded or run (no GPU needed).
+#include "annotations/abstract_function.h"
+#include "codegen/codegen.h"
+#include "compose/composable.h"
+#include "compose/compose.h"
+#include "compose/runner.h"
+#include "utils/error.h"
+
+#include "check.h"
+#include "library/array_device_annot.h"
+#include "library/device_host.h"
+#include "library/matrix_device_annot.h"
+
+#include <cstdlib>
+
+using namespace gern;
+
+static std::string libraryDir() {
+    const char *lib = std::getenv("GERN_TEST_LIBRARY");
+    return lib ? lib : "tests/cpp/library";
+}
+
+static std::string packageDir() {
+    const char *pkg = std::getenv("GERN_TEST_PACKAGE");
+    return pkg ? pkg : "gern_amd";
+}
+
+static bool compileOnly() {
+    const char *v = std::getenv("GERN_TEST_COMPILE_ONLY");
+    return v && v[0] == '1';
+}
+
+static std::string last_source;
+
+// Compiles the program; returns false when it was only compiled (no GPU run).
+static bool build(Runner &run, Composable program) {
+    if (compileOnly()) {
+        codegen::CodeGenerator cg;
+        last_source = cg.generate_code(program);
+        const std::string name = cg.getLaunchPlan().name_expression;
+        const std::string i1 = "-I" + libraryDir(), i2 = "-I" + packageDir();
+        const char *names[1] = {name.c_str()};
+        const char *opts[2] = {i1.c_str(), i2.c_str()};
+        size_t size = 0;
+        if (gern_hip_compile_only(last_source.c_str(), names, 1, opts, 2, "gfx950", &size) != 0) {
+            impl::hipCheck(1);
+        }
+        REQUIRE(size > 0);
+        return false;
+    }
+    Runner::Options o;
+    o.filename = "";
+    o.include = " -I " + libraryDir() + " -I " + packageDir();
+    run.compile(o);
+    last_source = run.getSource();
+    return true;
+}
+
+static AbstractDataTypePtr arrayDS(const std::string &name) {
+    return AbstractDataTypePtr(new const annot::ArrayGPU(name));
+}
+
+static void expect_offset(impl::ArrayGPU &a, impl::ArrayGPU &b, float off, int64_t n) {
+    std::vector<float> in = a.get(), out = b.get();
+    for (int64_t i = 0; i < n; i++) {
+        REQUIRE_EQ(out[i], in[i] + off);
+    }
+}
+
+// ---- test-gpu-array.cu ------------------------------------------------------------
+
+CASE("array.unmapped_runs_on_one_thread") {  // test-gpu-array.cu:16-76
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable step("step");
+    Composable program = Global(Tile(out["size"], step)(add_1(in, out)));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t step_val = 10;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}}));
+    expect_offset(a, b, 1, 10);
+    REQUIRE_THROWS_AS(run.evaluate({{in.getName(), &a}, {out.getName(), &b}}), error::UserError);
+    auto dummy = arrayDS("dummy_ds");
+    REQUIRE_THROWS_AS(run.evaluate({{in.getName(), &a}, {dummy.getName(), &b}}), error::UserError);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.tile_mapped_to_blocks") {  // test-gpu-array.cu:78-120
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable step("step");
+    Composable program = Global((Tile(out["size"], step) || Grid::Unit::BLOCK_X)(add_1(in, out)));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t step_val = 1;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}}));
+    expect_offset(a, b, 1, 10);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.tiles_mapped_to_blocks_and_threads") {  // test-gpu-array.cu:122-168
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable step("step"), blk("blk");
+    Composable program =
+        Global((Tile(out["size"], blk) || Grid::Unit::BLOCK_X)((Tile(out["size"], step) || Grid::Unit::THREAD_X)(add_1(in, out))));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t step_val = 1, blk_val = 1;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {blk.getName(), &blk_val}}));
+    expect_offset(a, b, 1, 10);
+    // a block of 5 elements, one thread each
+    blk_val = 5;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {blk.getName(), &blk_val}}));
+    expect_offset(a, b, 1, 10);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.register_arrays_fused") {  // test-gpu-array.cu:170-210
+    auto in = AbstractDataTypePtr(new const annot::ArrayStaticGPU("input_con"));
+    auto temp = AbstractDataTypePtr(new const annot::ArrayStaticGPU("temp", true));
+    auto out = AbstractDataTypePtr(new const annot::ArrayStaticGPU("output_con"));
+    annot::Add1GPUTemplate add_1;
+    Variable step("step"), blk("blk");
+    Composable program = Global((Tile(out["size"], blk) || Grid::Unit::BLOCK_X)(
+        (Tile(out["size"], step.bind(1)) || Grid::Unit::THREAD_X)(add_1(in, temp), add_1(temp, out))));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t blk_val = 5;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {blk.getName(), &blk_val}}));
+    expect_offset(a, b, 2, 10);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.repeated_units") {  // test-gpu-array.cu:212-254
+    auto in = AbstractDataTypePtr(new const annot::ArrayStaticGPU("input_con"));
+    auto temp = AbstractDataTypePtr(new const annot::ArrayStaticGPU("temp", true));
+    auto out = AbstractDataTypePtr(new const annot::ArrayStaticGPU("output_con"));
+    annot::Add1GPUTemplate add_1;
+    Variable step("step"), step2("step2"), step3("step3"), blk("blk");
+    Composable program = Global((Tile(out["size"], blk.bind(8)) || Grid::Unit::BLOCK_X)(
+        (Tile(out["size"], step.bind(4)) || Grid::Unit::BLOCK_X)((Tile(out["size"], step2.bind(2)) || Grid::Unit::THREAD_X)(
+            (Tile(out["size"], step3.bind(1)) || Grid::Unit::THREAD_Y)(
+                (Tile(out["size"], step3.bind(1)) || Grid::Unit::THREAD_X)(add_1(in, temp), add_1(temp, out)))))));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(16), b(16);
+    a.ascending();
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}}));
+    expect_offset(a, b, 2, 16);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.reduction_hoisted_out_of_mapped_loops") {  // test-gpu-array.cu:256-297
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::reductionGPU reduce;
+    Variable step("step"), blk("blk"), k("k"), k2("k2");
+    Composable program = Global(Tile(out["size"], k2.bind(10))(Reduce(k, step.bind(5))(
+        (Tile(out["size"], step.bind(5)) || Grid::Unit::BLOCK_X)(
+            (Tile(out["size"], blk.bind(1)) || Grid::Unit::THREAD_X)(Reduce(k, blk.bind(1))(reduce(in, out, k)))))));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t k_val = 10;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {k.getName(), &k_val}}));
+    std::vector<float> r = b.get();
+    for (int i = 0; i < 10; i++) {
+        REQUIRE_EQ(r[i], 45.0f);
+    }
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.tile_mapped_to_wavefronts") {
+    // Specific to this backend: a WARP unit is a 64-lane wavefront, so the
+    // index expression divides threadIdx.x by 64 and the block grows by 64
+    // threads per tile.  All 64 lanes of a wavefront compute the same tile.
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable step("step"), blk("blk");
+    Composable program =
+        Global((Tile(out["size"], blk) || Grid::Unit::BLOCK_X)((Tile(out["size"], step) || Grid::Unit::WARP_X)(add_1(in, out))));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("/ 64") != std::string::npos);
+    REQUIRE(last_source.find("/ 32") == std::string::npos);
+    if (!ran) {
+        return;
+    }
+    impl::ArrayGPU a(12), b(12);
+    a.ascending();
+    int64_t step_val = 2, blk_val = 6;  // 2 blocks x 3 wavefronts
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {blk.getName(), &blk_val}}));
+    expect_offset(a, b, 1, 12);
+    a.destroy();
+    b.destroy();
+}
+
+// ---- test-set-grid.cu -----------------------------------------------------------------
+
+CASE("set_grid.only_dimensions_in_scope") {  // test-set-grid.cu:15-44
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::AddArrayThreads add_1;
+    Variable step("step");
+    REQUIRE_NOTHROW(Global(Tile(out["size"], step)(add_1(in, out))));
+    REQUIRE_NOTHROW(Global(Tile(out["size"], step)(add_1(in, out)), {{Grid::Dim::BLOCK_DIM_X, step}}));
+    REQUIRE_THROWS_AS(Global(Tile(out["size"], step)(add_1(in, out)), {{Grid::Dim::BLOCK_DIM_Y, step}}), error::UserError);
+}
+
+static void set_grid_run(bool separate_variable) {  // test-set-grid.cu:46-136
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::AddArrayThreads add_1;
+    Variable step("step"), num_threads("num_threads");
+    Composable program =
+        Global(Tile(out["size"], step)(add_1(in, out)), {{Grid::Dim::BLOCK_DIM_X, separate_variable ? num_threads : step}});
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t step_val = 5, threads_val = 5;
+    std::map<std::string, void *> args = {{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}};
+    if (separate_variable) {
+        args[num_threads.getName()] = &threads_val;
+    }
+    REQUIRE_NOTHROW(run.evaluate(args));
+    expect_offset(a, b, 1, 10);
+    if (separate_variable) {
+        // the function assumes blockDim.x >= step: the launch is refused on the host
+        threads_val = 2;
+        REQUIRE_THROWS_AS(run.evaluate(args), error::UserError);
+    }
+    a.destroy();
+    b.destroy();
+}
+
+CASE("set_grid.block_size_from_tile_variable") {
+    set_grid_run(false);
+}
+
+CASE("set_grid.block_size_from_own_variable_and_assumption") {
+    set_grid_run(true);
+}
+
+// ---- test-dynamic-shared.cu ----------------------------------------------------------------
+
+class LdsManager : public grid::SharedMemoryManager {
+public:
+    explicit LdsManager(Variable smem_size)
+        : grid::SharedMemoryManager(
+              FunctionCall{"gernels::lds_init", {smem_size}, {}, Parameter(), LaunchArguments(), LaunchArguments(), DEVICE},
+              {"gernels/lds_alloc.h"}) {
+    }
+};
+
+static void dynamic_lds_run(bool with_manager) {  // test-dynamic-shared.cu:15-105
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable step("step"), smem_size("smem_size");
+    Composable program = with_manager ? Global(Tile(out["size"], step)(add_1(in, out)), {}, smem_size, LdsManager(smem_size)) :
+                                        Global(Tile(out["size"], step)(add_1(in, out)), {}, smem_size);
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t step_val = 10, smem_val = 1024;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {smem_size.getName(), &smem_val}}));
+    expect_offset(a, b, 1, 10);
+    // more LDS than a gfx950 workgroup can have (160 KB) is refused on the host
+    smem_val = 200 * 1024;
+    REQUIRE_THROWS_AS(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {smem_size.getName(), &smem_val}}),
+                      error::UserError);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("dynamic_lds.size_only") {
+    dynamic_lds_run(false);
+}
+
+CASE("dynamic_lds.with_allocator_init") {
+    dynamic_lds_run(true);
+}
+
+CASE("dynamic_lds.tiles_staged_into_lds") {  // test-dynamic-shared.cu:107-175
+    auto in = AbstractDataTypePtr(new const annot::MatrixGPUStageSmem("input_con"));
+    auto out = AbstractDataTypePtr(new const annot::MatrixGPUStageSmem("output_con"));
+    annot::MatrixAddGPUBlocks add_blocks;
+    Variable l_x("l_x"), l_y("l_y"), smem_size("smem_size"), thread_x("thread_x"), thread_y("thread_y");
+    Composable program =
+        Global((Tile(out["row"], l_x) || Grid::Unit::BLOCK_X)((Tile(out["col"], l_y) || Grid::Unit::BLOCK_Y)(add_blocks(in, out))),
+               {{Grid::Dim::BLOCK_DIM_X, thread_x}, {Grid::Dim::BLOCK_DIM_Y, thread_y}}, smem_size, LdsManager(smem_size));
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    const int64_t rows = 4, cols = 8;
+    impl::MatrixGPU a(rows, cols, cols), b(rows, cols, cols);
+    a.ascending();
+    int64_t lx = 4, ly = 2, tx = 1, ty = 2, smem = 1024;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {l_x.getName(), &lx}, {l_y.getName(), &ly},
+                                  {smem_size.getName(), &smem}, {thread_x.getName(), &tx}, {thread_y.getName(), &ty}}));
+    std::vector<float> r = b.get(), src = a.get();
+    for (int64_t i = 0; i < rows * cols; i++) {
+        REQUIRE_EQ(r[i], src[i] + 1.0f);
+    }
+    a.destroy();
+    b.destroy();
+}
+
+// ---- test-gpu-matrix.cu ----------------------------------------------------------------------
+
+static void matrix_add(int mapped) {  // test-gpu-matrix.cu:15-190
+    auto in = AbstractDataTypePtr(new const annot::MatrixGPU("input_con"));
+    auto out = AbstractDataTypePtr(new const annot::MatrixGPU("output_con"));
+    annot::MatrixAddGPU add;
+    Variable l_x("l_x"), l_y("l_y");
+    Composable program;
+    if (mapped == 0) {
+        program = Global(Tile(out["row"], l_x)(Tile(out["col"], l_y)(add(in, out))));
+    } else if (mapped == 1) {
+        program = Global((Tile(out["row"], l_x) || Grid::Unit::BLOCK_X)(Tile(out["col"], l_y)(add(in, out))));
+    } else {
+        program = Global((Tile(out["row"], l_x) || Grid::Unit::BLOCK_X)((Tile(out["col"], l_y) || Grid::Unit::BLOCK_Y)(add(in, out))));
+    }
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::MatrixGPU a(10, 10, 10), b(10, 10, 10);
+    a.fill(2.0f);
+    int64_t lx = 5, ly = 5;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {l_x.getName(), &lx}, {l_y.getName(), &ly}}));
+    for (float v : b.get()) {
+        REQUIRE_EQ(v, 3.0f);
+    }
+    a.fill(7.0f);
+    ly = 2;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {l_x.getName(), &lx}, {l_y.getName(), &ly}}));
+    for (float v : b.get()) {
+        REQUIRE_EQ(v, 8.0f);
+    }
+    a.destroy();
+    b.destroy();
+}
+
+CASE("matrix.add_unmapped") {
+    matrix_add(0);
+}
+
+CASE("matrix.add_rows_on_blocks") {
+    matrix_add(1);
+}
+
+CASE("matrix.add_rows_and_columns_on_blocks") {
+    matrix_add(2);
+}
+
+CHECK_MAIN()
