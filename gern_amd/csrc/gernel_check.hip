@@ -83,7 +83,7 @@ template __global__ void check_gemm_f32<128, 128, 4096>(gernels::MatrixF32, gern
 #include "gernels/qk_softmax.h"
 
 template<int64_t N, int64_t D>
-__global__ void __launch_bounds__(256) check_qk_softmax(gernels::MatrixBF16 Q, gernels::MatrixBF16 K, gernels::MatrixF32 S,
+__global__ void __launch_bounds__(64 * gernels::qk_waves(N)) check_qk_softmax(gernels::MatrixBF16 Q, gernels::MatrixBF16 K, gernels::MatrixF32 S,
                                                         float scale) {
     const int64_t x = blockIdx.x * 16;
     auto q = Q.template view<16, D>(x, 0);

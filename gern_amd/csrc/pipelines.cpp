@@ -65,6 +65,11 @@ struct gern_pipeline_s {
 
 namespace {
 
+// The rule of gernels/qk_softmax.h (qk_waves): wavefronts per row block.
+int64_t qkWaves(int64_t n) {
+    return (n >= 4096 && n % 1024 == 0) ? 16 : (n >= 2048 && n % 512 == 0) ? 8 : 4;
+}
+
 // Generates (and, unless compile-only, loads) the program.
 int finish(gern_pipeline_s *p, Composable program, int flags) {
     const std::string include = "-I " + packageDir();
@@ -406,7 +411,9 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
                 qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), max_row[width](row_max, logits),
                 sub(row_max, logits, shifted), ex(shifted, expd), sum_row[width](row_sum, expd),
                 div(row_sum, expd, S))),
-            {{Grid::BLOCK_DIM_X, threads.bind(256)}});
+            // gernels/qk_softmax.h, qk_waves(): more wavefronts share a row
+            // block as it gets wider.
+            {{Grid::BLOCK_DIM_X, threads.bind(64 * qkWaves(max_keys))}});
         int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
         if (rc != 0) {
             return rc;

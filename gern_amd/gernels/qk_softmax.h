@@ -1,15 +1,21 @@
 // Fused S = softmax_rows(scale * Q K^T) for bf16 Q (M x D) and K (N x D).
 //
-// One workgroup (four wavefronts) owns 16 rows of S and ALL N <= 4096 columns,
-// held as MFMA accumulators: wavefront w owns columns [w*N/4, (w+1)*N/4), as
-// N/256 groups of 64 columns, each group four v_mfma_f32_16x16x32_bf16 tiles.
+// One workgroup of NW wavefronts owns 16 rows of S and ALL N <= 4096 columns,
+// held as MFMA accumulators: wavefront w owns columns [w*N/NW, (w+1)*N/NW), as
+// groups of 64 columns, each group four v_mfma_f32_16x16x32_bf16 tiles.
 // Inside a group, tile t / lane column j stands for key 4*j + t, so that the
 // four tiles of a group give every lane FOUR CONSECUTIVE columns of S and a row
 // of the block is stored with 16-byte stores, 256 contiguous bytes per sixteen
 // lanes.  The logits never leave registers: row maximum and row sum are reduced
-// inside the 16-lane DPP rows that share an S row, then across the four
-// wavefronts through 256 bytes of LDS.  S is written once; Q and K (1 MiB each,
-// L2-resident) are the only reads.
+// inside the 16-lane DPP rows that share an S row, then across the wavefronts
+// through a few hundred bytes of LDS (one barrier per reduction).  S is
+// written once, with streaming stores; Q and K (1 MiB each, L2-resident) are
+// the only reads.
+//
+// NW grows with N (16 wavefronts for 4096 keys): S has only M/16 row blocks,
+// so the columns of a block must be spread over as many wavefronts as a CU can
+// hold for the chip to be busy, and 64 accumulators per lane leave room for
+// four wavefronts per SIMD.
 //
 // The reference has nothing like this (no bf16, no matrix-core path, no fused
 // GEMM -> softmax); the softmax stages reuse the names and argument order of
@@ -24,16 +30,30 @@ namespace gernels {
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+// Wavefronts per workgroup for a row block of N columns; the host sizes the
+// launch with the same rule (threads = 64 * qk_waves(N)).
+#ifndef GERN_QK_WAVES
+constexpr int qk_waves(int64_t n) {
+    return (n >= 4096 && n % 1024 == 0) ? 16 : (n >= 2048 && n % 512 == 0) ? 8 : 4;
+}
+#else
+constexpr int qk_waves(int64_t) {
+    return GERN_QK_WAVES;
+}
+#endif
+
 // 16 x N logits / probabilities, distributed over the workgroup as described
 // above: acc[g][t][i] is row 4*(lane/16) + i, column
-// wave*(N/4) + 64*g + 4*(lane%16) + t.
+// wave*(N/NW) + 64*g + 4*(lane%16) + t.
 template<int64_t R, int64_t N>
 struct RowBlock {
     static_assert(R == 16, "a row block is one MFMA tile high");
-    static_assert(N % 256 == 0 && N <= 4096, "four wavefronts x 64-column groups, at most 256 accumulators");
+    static constexpr int NW = qk_waves(N);
+    static_assert(N % (64 * NW) == 0 && N <= 4096, "wavefronts x 64-column groups, at most 4096 columns");
     static constexpr int64_t rows = R;
     static constexpr int64_t cols = N;
-    static constexpr int G = (int)(N / 256);
+    static constexpr int64_t wave_cols = N / NW;
+    static constexpr int G = (int)(N / (64 * NW));
     f32x4_t acc[G][4];
 
     __device__ __forceinline__ void destroy() {
@@ -70,7 +90,7 @@ template<int64_t R, int64_t N>
 __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y, const RowBlock<R, N> &t) const {
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
-    const int64_t c0 = y + (int64_t)w * (N / 4) + 4 * (lane % 16);
+    const int64_t c0 = y + (int64_t)w * RowBlock<R, N>::wave_cols + 4 * (lane % 16);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int64_t rr = x + 4 * (lane / 16) + i;
@@ -84,7 +104,7 @@ __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y,
             const int64_t cc = c0 + 64 * g;
             const float4 val = make_float4(t.acc[g][0][i], t.acc[g][1][i], t.acc[g][2][i], t.acc[g][3][i]);
             if (vec_ok && cc + 3 < col) {
-                *reinterpret_cast<float4 *>(p + cc) = val;
+                store_streaming(p + cc, val);
             } else {
                 if (cc + 0 < col) p[cc + 0] = val.x;
                 if (cc + 1 < col) p[cc + 1] = val.y;
@@ -122,7 +142,7 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
     for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const int64_t key = (int64_t)w * (N / 4) + 64 * g + 4 * (lane % 16) + t;
+            const int64_t key = (int64_t)w * RowBlock<R, N>::wave_cols + 64 * g + 4 * (lane % 16) + t;
             const bool ok = key < K.rows;
             f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -139,7 +159,7 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
         // per-lane, per-tile property.
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const int64_t key = (int64_t)w * (N / 4) + 64 * g + 4 * (lane % 16) + t;
+            const int64_t key = (int64_t)w * RowBlock<R, N>::wave_cols + 64 * g + 4 * (lane % 16) + t;
             if (key >= K.rows) {
                 S.acc[g][t] = f32x4_t{-__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf(),
                                       -__builtin_huge_valf()};
@@ -150,37 +170,61 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
 
 namespace detail {
 
-// Reduces over the 16 lanes of a DPP row (the lanes that share S rows), then
-// over the four wavefronts.
-template<typename Op>
-__device__ __forceinline__ float row_block_reduce(float x, float *lds, int slot) {
-    x = Op::apply(x, dpp_move<0xB1>(x));   // quad_perm [1,0,3,2]
-    x = Op::apply(x, dpp_move<0x4E>(x));   // quad_perm [2,3,0,1]
-    x = Op::apply(x, dpp_move<0x141>(x));  // row_half_mirror
-    x = Op::apply(x, dpp_move<0x140>(x));  // row_mirror
+// Reduces the four row values of a lane over the 16 lanes of a DPP row (the
+// lanes that share S rows), then over the NW wavefronts through `lds`
+// (16 rows x NW floats; the two reductions of a softmax use different buffers,
+// so one barrier each is enough).
+template<typename Op, int NW>
+__device__ __forceinline__ void row_block_reduce(float (&x)[4], float *lds) {
+    const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
-    lds[w * 16 + slot] = x;  // all 16 lanes of the row write the same value
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float v = x[i];
+        v = Op::apply(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+        v = Op::apply(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+        v = Op::apply(v, dpp_move<0x141>(v));  // row_half_mirror
+        v = Op::apply(v, dpp_move<0x140>(v));  // row_mirror
+        x[i] = v;
+    }
+    if (lane % 16 == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            lds[(4 * (lane / 16) + i) * NW + w] = x[i];
+        }
+    }
     __syncthreads();
-    float r = Op::apply(Op::apply(lds[slot], lds[16 + slot]), Op::apply(lds[32 + slot], lds[48 + slot]));
-    __syncthreads();
-    return r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const f32x4_t *row = reinterpret_cast<const f32x4_t *>(lds + (4 * (lane / 16) + i) * NW);
+        float r = Op::identity();
+#pragma unroll
+        for (int q = 0; q < NW / 4; q++) {
+            const f32x4_t part = row[q];
+            r = Op::apply(Op::apply(r, part[0]), Op::apply(part[1], Op::apply(part[2], part[3])));
+        }
+        x[i] = r;
+    }
 }
 
 template<typename Op, int64_t R, int64_t N>
-__device__ __forceinline__ void reduce_row_block(RowStat<R> &out, const RowBlock<R, N> &in) {
-    __shared__ float scratch[64];
-    const int lane = lane_id();
+__device__ __forceinline__ void reduce_row_block(RowStat<R> &out, const RowBlock<R, N> &in, float *lds) {
+    float acc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        float acc = Op::identity();
+        acc[i] = Op::identity();
 #pragma unroll
         for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                acc = Op::apply(acc, in.acc[g][t][i]);
+                acc[i] = Op::apply(acc[i], in.acc[g][t][i]);
             }
         }
-        out.v[i] = row_block_reduce<Op>(acc, scratch, 4 * (lane / 16) + i);
+    }
+    row_block_reduce<Op, RowBlock<R, N>::NW>(acc, lds);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        out.v[i] = acc[i];
     }
 }
 
@@ -188,12 +232,14 @@ __device__ __forceinline__ void reduce_row_block(RowStat<R> &out, const RowBlock
 
 template<int64_t stride = 64, int64_t R, int64_t N>
 __device__ __forceinline__ void max_row(RowStat<R> &out, const RowBlock<R, N> &in) {
-    detail::reduce_row_block<MaxOp>(out, in);
+    __shared__ __attribute__((aligned(16))) float max_scratch[16 * RowBlock<R, N>::NW];
+    detail::reduce_row_block<MaxOp>(out, in, max_scratch);
 }
 
 template<int64_t stride = 64, int64_t R, int64_t N>
 __device__ __forceinline__ void sum_row(RowStat<R> &out, const RowBlock<R, N> &in) {
-    detail::reduce_row_block<SumOp>(out, in);
+    __shared__ __attribute__((aligned(16))) float sum_scratch[16 * RowBlock<R, N>::NW];
+    detail::reduce_row_block<SumOp>(out, in, sum_scratch);
 }
 
 template<int64_t R, int64_t N>
@@ -216,10 +262,9 @@ __device__ __forceinline__ void exp_matrix(const RowBlock<R, N> &in, RowBlock<R,
     for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                out.acc[g][t][i] = expf(in.acc[g][t][i]);
-            }
+            const f32x4_t a = in.acc[g][t];
+            const float4 e = exp4(make_float4(a[0], a[1], a[2], a[3]));
+            out.acc[g][t] = f32x4_t{e.x, e.y, e.z, e.w};
         }
     }
 }
@@ -237,7 +282,7 @@ __device__ __forceinline__ void divide_vec(const RowStat<R> &vec, const RowBlock
         for (int t = 0; t < 4; t++) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                out.acc[g][t][i] = div_by(in.acc[g][t][i], vec.v[i], rcp[i]);
+                out.acc[g][t][i] = in.acc[g][t][i] * rcp[i];
             }
         }
     }

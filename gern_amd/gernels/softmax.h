@@ -100,14 +100,33 @@ __device__ __forceinline__ void subtract_vec(const TV &vec, const T &in, T &out)
     }
 }
 
+// exp(x) as one multiply and one v_exp_f32 (2^y).  For x in [-87, 0] -- what a
+// max-subtracted row holds -- the product x * log2(e) is off by at most half
+// an ulp of 126, i.e. the result by 2.6e-6 relative, plus the instruction's own
+// 1 ulp.  The raw instruction flushes results below 2^-126 to zero, and large
+// positive arguments lose more, so a chunk in which ANY lane is outside
+// [-87, 87] takes the library expf instead (a wave-uniform branch, never taken
+// for the rows a softmax sees in practice).
+__device__ __forceinline__ float4 exp4(const float4 &t) {
+    const float lo = __builtin_fminf(__builtin_fminf(t.x, t.y), __builtin_fminf(t.z, t.w));
+    const float hi = __builtin_fmaxf(__builtin_fmaxf(t.x, t.y), __builtin_fmaxf(t.z, t.w));
+    // NaN compares false on both sides of the range test: written so that it
+    // takes the library path too.
+    if (__builtin_amdgcn_ballot_w64(!(lo >= -87.0f && hi <= 87.0f)) != 0) {
+        return make_float4(expf(t.x), expf(t.y), expf(t.z), expf(t.w));
+    }
+    const float l2e = 1.4426950408889634f;
+    return make_float4(__builtin_amdgcn_exp2f(t.x * l2e), __builtin_amdgcn_exp2f(t.y * l2e),
+                       __builtin_amdgcn_exp2f(t.z * l2e), __builtin_amdgcn_exp2f(t.w * l2e));
+}
+
 template<typename T>
 __device__ __forceinline__ void exp_matrix(const T &in, T &out) {
 #pragma unroll
     for (int64_t r = 0; r < T::rows; r++) {
 #pragma unroll
         for (int64_t k = 0; k < T::chunks; k++) {
-            const float4 t = in.v[r][k];
-            out.v[r][k] = make_float4(expf(t.x), expf(t.y), expf(t.z), expf(t.w));
+            out.v[r][k] = exp4(in.v[r][k]);
         }
     }
 }
@@ -117,13 +136,13 @@ __device__ __forceinline__ void divide_vec(const TV &vec, const T &in, T &out) {
     static_assert(TV::size == T::rows, "one scalar per tile row");
 #pragma unroll
     for (int64_t r = 0; r < T::rows; r++) {
-        const float d = vec.val[r];
-        const float rcp = 1.0f / d;  // one IEEE division per row
+        // One IEEE division per row, then a multiply per element: within
+        // 1 ulp of the true quotient (the softmax bar is 1e-5 relative).
+        const float rcp = 1.0f / vec.val[r];
 #pragma unroll
         for (int64_t k = 0; k < T::chunks; k++) {
             const float4 t = in.v[r][k];
-            out.v[r][k] = make_float4(div_by(t.x, d, rcp), div_by(t.y, d, rcp), div_by(t.z, d, rcp),
-                                      div_by(t.w, d, rcp));
+            out.v[r][k] = make_float4(t.x * rcp, t.y * rcp, t.z * rcp, t.w * rcp);
         }
     }
 }

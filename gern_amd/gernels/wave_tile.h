@@ -40,6 +40,13 @@ struct WaveVec {
     }
 };
 
+// 16-byte streaming store (the nontemporal builtin wants a native vector).
+__device__ __forceinline__ void store_streaming(float *p, const float4 &v) {
+    typedef float f32x4_native __attribute__((ext_vector_type(4)));
+    const f32x4_native q = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(q, reinterpret_cast<f32x4_native *>(p));
+}
+
 template<int64_t R, int64_t C>
 __device__ __forceinline__ WaveTile<R, C> allocate_wave_tile() {
     return WaveTile<R, C>();
@@ -155,7 +162,11 @@ struct MatrixF32 {
                 const int64_t cc = y + lc;
                 const float4 val = t.v[r][k];
                 if (vec_ok && lc + 3 < C && cc + 3 < col) {
-                    *reinterpret_cast<float4 *>(p + lc) = val;
+                    // A result tile is written once and never read back by
+                    // the kernel: a streaming (nontemporal) store keeps it
+                    // from displacing the input rows that neighbouring tiles
+                    // are about to re-read from L2.
+                    store_streaming(p + lc, val);
                 } else {
                     if (lc + 0 < C && cc + 0 < col) p[lc + 0] = val.x;
                     if (lc + 1 < C && cc + 1 < col) p[lc + 1] = val.y;
