@@ -144,5 +144,29 @@ private:
     Variable scale{"scale", Datatype::Float32};
 };
 
+// divide_vec for row blocks: a block spans ALL columns of its rows (the row
+// statistics are those of whole rows), so the output may not be wider than
+// one tile.  The launch is refused otherwise, and the generated kernel knows
+// that its loop over column tiles runs once.
+class DivideVecWholeRows : public DivideVec {
+public:
+    using DivideVec::DivideVec;
+    Annotation getAnnotation() override {
+        Variable x("x");
+        Variable y("y");
+        Variable l_x("l_x", Datatype::Int64, true);
+        Variable l_y("l_y", Datatype::Int64, true);
+        return Tileable(x = Expr(0), ADTMember(output, "row", false), l_x,
+                        Tileable(y = Expr(0), ADTMember(output, "col", false), l_y,
+                                 Produces::Subset(output, {x, y, l_x, l_y}),
+                                 Consumes::Subsets(SubsetObjMany({
+                                     SubsetObj(input, {x, y, l_x, l_y}),
+                                     SubsetObj(vec, {x, l_x}),
+                                 }))))
+            .occupies({Grid::Unit::THREAD_X_IN_WRAPS})
+            .assumes(Constraint(ADTMember(output, "col", false) <= l_y));
+    }
+};
+
 }  // namespace annot
 }  // namespace gern

@@ -67,7 +67,7 @@ namespace {
 
 // The rule of gernels/qk_softmax.h (qk_waves): wavefronts per row block.
 int64_t qkWaves(int64_t n) {
-    return (n >= 4096 && n % 1024 == 0) ? 16 : (n >= 2048 && n % 512 == 0) ? 8 : 4;
+    return (n >= 2048 && n % 512 == 0) ? 8 : 4;
 }
 
 // Generates (and, unless compile-only, loads) the program.
@@ -404,7 +404,7 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
         annot::SubtractVec sub{row_max, logits, shifted};
         annot::ExpMatrix ex{shifted, expd};
         annot::SumRow sum_row{expd, row_sum};
-        annot::DivideVec div{row_sum, expd, S};
+        annot::DivideVecWholeRows div{row_sum, expd, S};
         std::map<std::string, Variable> width{{"ncol", keys.bind(max_keys)}};
         Composable program = Global(
             (Tile(S["row"], rows.bind(16)) || Grid::BLOCK_X)(Tile(S["col"], keys.bind(max_keys))(

@@ -12,10 +12,11 @@
 // written once, with streaming stores; Q and K (1 MiB each, L2-resident) are
 // the only reads.
 //
-// NW grows with N (16 wavefronts for 4096 keys): S has only M/16 row blocks,
-// so the columns of a block must be spread over as many wavefronts as a CU can
-// hold for the chip to be busy, and 64 accumulators per lane leave room for
-// four wavefronts per SIMD.
+// NW grows with N (8 wavefronts from 2048 keys on): S has only M/16 row
+// blocks, so the columns of a block are spread over several wavefronts for the
+// chip to be busy; 128 accumulators per lane leave room for two wavefronts per
+// SIMD (16 wavefronts with 64 accumulators each measured slower: the
+// compiler spills at 128 registers).
 //
 // The reference has nothing like this (no bf16, no matrix-core path, no fused
 // GEMM -> softmax); the softmax stages reuse the names and argument order of
@@ -34,7 +35,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // launch with the same rule (threads = 64 * qk_waves(N)).
 #ifndef GERN_QK_WAVES
 constexpr int qk_waves(int64_t n) {
-    return (n >= 4096 && n % 1024 == 0) ? 16 : (n >= 2048 && n % 512 == 0) ? 8 : 4;
+    return (n >= 2048 && n % 512 == 0) ? 8 : 4;
 }
 #else
 constexpr int qk_waves(int64_t) {
@@ -115,8 +116,9 @@ __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y,
     }
 }
 
-// S = scale * Q K^T for the 16 rows of Q in view; columns past the last key
-// get -inf so that they vanish from the softmax.
+// S = log2(e) * scale * Q K^T for the 16 rows of Q in view (log2 units, see
+// exp_matrix below); columns past the last key get -inf so that they vanish
+// from the softmax.
 template<int64_t R, int64_t N, int64_t D>
 __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false> &Q, const GlobalView<N, D, uint16_t, false> &K,
                                           RowBlock<R, N> &S, float scale) {
@@ -138,22 +140,37 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
             q[s] = __builtin_bit_cast(bf16x8_t, v);
         }
     }
+    // K is read with lanes 4j .. 4j+3 on the four 16-byte pieces of ONE key's
+    // 64 bytes (sixteen keys per load), so that each group of four lanes
+    // touches a single cache line: the vector cache looks up one line per
+    // cycle, and the layout the MFMA wants (lane l: key l%16, piece l/16) would
+    // make every lane of a quad hit a different line, a quarter of the rate.
+    // The pieces then move to the lanes that feed the MFMA with ds_bpermute
+    // (lane l takes from lane 4*(l%16) + l/16), which costs no LDS space.
+    const int take_from = 4 * (4 * (lane % 16) + lane / 16);
+    // The logits are kept in log2 units (scale * log2(e) folded into one
+    // multiply), so that the exp stage is a bare v_exp_f32.
+    const float to_log2 = scale * 1.4426950408889634f;
 #pragma unroll
     for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const int64_t key = (int64_t)w * RowBlock<R, N>::wave_cols + 64 * g + 4 * (lane % 16) + t;
-            const bool ok = key < K.rows;
+            const int64_t load_key = (int64_t)w * RowBlock<R, N>::wave_cols + 64 * g + 4 * (lane / 4) + t;
+            const bool ok = load_key < K.rows;
             f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < KS; s++) {
                 uint4 v = make_uint4(0u, 0u, 0u, 0u);
                 if (ok) {
-                    v = *reinterpret_cast<const uint4 *>(K.data + key * K.lda + s * 32 + k_off);
+                    v = *reinterpret_cast<const uint4 *>(K.data + load_key * K.lda + s * 32 + 8 * (lane % 4));
                 }
+                v.x = (uint32_t)__builtin_amdgcn_ds_bpermute(take_from, (int)v.x);
+                v.y = (uint32_t)__builtin_amdgcn_ds_bpermute(take_from, (int)v.y);
+                v.z = (uint32_t)__builtin_amdgcn_ds_bpermute(take_from, (int)v.z);
+                v.w = (uint32_t)__builtin_amdgcn_ds_bpermute(take_from, (int)v.w);
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(q[s], __builtin_bit_cast(bf16x8_t, v), acc, 0, 0, 0);
             }
-            S.acc[g][t] = acc * scale;
+            S.acc[g][t] = acc * to_log2;
         }
         // The column a lane holds in tile t is its own key, so validity is a
         // per-lane, per-tile property.
@@ -256,6 +273,10 @@ __device__ __forceinline__ void subtract_vec(const RowStat<R> &vec, const RowBlo
     }
 }
 
+// A row block holds logits in log2 units, so exp is 2^x: one v_exp_f32 per
+// element.  Its arguments are <= 0 here (a row maximum has been subtracted);
+// results below 2^-126 come out as 0, i.e. probabilities that fp32 could only
+// hold as denormals are flushed to zero.
 template<int64_t R, int64_t N>
 __device__ __forceinline__ void exp_matrix(const RowBlock<R, N> &in, RowBlock<R, N> &out) {
 #pragma unroll
@@ -263,8 +284,8 @@ __device__ __forceinline__ void exp_matrix(const RowBlock<R, N> &in, RowBlock<R,
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const f32x4_t a = in.acc[g][t];
-            const float4 e = exp4(make_float4(a[0], a[1], a[2], a[3]));
-            out.acc[g][t] = f32x4_t{e.x, e.y, e.z, e.w};
+            out.acc[g][t] = f32x4_t{__builtin_amdgcn_exp2f(a[0]), __builtin_amdgcn_exp2f(a[1]),
+                                    __builtin_amdgcn_exp2f(a[2]), __builtin_amdgcn_exp2f(a[3])};
         }
     }
 }

@@ -425,8 +425,11 @@ public:
         } else if (!device) {
             line(indent, "assert(" + gen(c) + ");");
         } else {
-            // Device code never traps; the Runner checks this before launch.
-            gen(c);
+            // Device code never traps; the Runner checks this before launch
+            // and refuses the launch when it does not hold.  The kernel may
+            // therefore rely on it: the compiler is told, which lets it, for
+            // one, see that a loop over a single tile runs once.
+            line(indent, "__builtin_assume(" + gen(c) + ");");
             host_asserts.push_back(c);
         }
     }

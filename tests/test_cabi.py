@@ -86,3 +86,49 @@ def test_runtime_reports_compile_errors():
     buf = C.create_string_buffer(4096)
     hip.gern_hip_last_error(buf, 4096)
     assert b"error" in buf.value
+
+
+def _kernel_notes(tmp_path, make_pipeline):
+    """Compiles a pipeline with the run-time compiler (no GPU needed) and reads the resource
+    usage the compiler recorded in the code object."""
+    import shutil
+    import subprocess
+    readelf = shutil.which("llvm-readelf") or "/opt/rocm/llvm/bin/llvm-readelf"
+    if not os.path.exists(readelf):
+        pytest.skip("llvm-readelf not available")
+    os.environ["GERN_HIP_KEEP_DIR"] = str(tmp_path)
+    try:
+        make_pipeline()
+    finally:
+        del os.environ["GERN_HIP_KEEP_DIR"]
+    kernels = []
+    for f in sorted(tmp_path.glob("*.hsaco")):
+        out = subprocess.run([readelf, "--notes", str(f)], stdout=subprocess.PIPE, text=True, check=True).stdout
+        cur = {}
+        for line in out.splitlines():
+            line = line.strip().lstrip("- ")
+            for key in (".name", ".vgpr_count", ".agpr_count", ".vgpr_spill_count", ".private_segment_fixed_size"):
+                if line.startswith(key + ":"):
+                    val = line.split(":", 1)[1].strip()
+                    cur[key] = val if key == ".name" else int(val)
+            if ".name" in cur and ".vgpr_spill_count" in cur and ".private_segment_fixed_size" in cur and ".vgpr_count" in cur:
+                kernels.append(cur)
+                cur = {}
+    assert kernels, "no kernel metadata found"
+    return kernels
+
+
+@pytest.mark.parametrize("name,make", [
+    ("blur_xyx", lambda: gern_amd.BlurChain("xyx", tile_rows=4, flags=gern_amd.COMPILE_ONLY)),
+    ("softmax_4096", lambda: gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY)),
+    ("gemm_f32", lambda: gern_amd.Gemm("f32", overwrite=True, flags=gern_amd.COMPILE_ONLY)),
+    ("gemm_bf16", lambda: gern_amd.Gemm("bf16", overwrite=True, flags=gern_amd.COMPILE_ONLY)),
+    ("gemm_bf16_accumulate", lambda: gern_amd.Gemm("bf16", flags=gern_amd.COMPILE_ONLY)),
+    ("qk_softmax_4096", lambda: gern_amd.QKSoftmax(128, 4096, flags=gern_amd.COMPILE_ONLY)),
+])
+def test_headline_kernels_use_no_scratch_memory(tmp_path, name, make):
+    # A kernel that spills registers, or keeps an array on the stack, writes to
+    # HBM on every iteration: once, that made the bf16 GEMM move 11x its result.
+    for k in _kernel_notes(tmp_path, make):
+        assert k[".vgpr_spill_count"] == 0, (name, k)
+        assert k[".private_segment_fixed_size"] == 0, (name, k)
