@@ -190,9 +190,181 @@ constexpr int64_t mfma_lds_bytes() {
     return 2 * (BM + BN) * kMfmaRowBytes;
 }
 
+namespace detail {
+
+// The fast bf16 path: 256 x 256 tile, eight wavefronts, whole tiles only.
+//
+// Wavefronts 0-3 (one per SIMD) move A, wavefronts 4-7 move B, and the two
+// groups run half a stage out of phase: while one group issues its MFMAs the
+// other writes the next stage into LDS and issues the global loads of the stage
+// after it, so every SIMD always holds one wavefront that computes and one
+// that moves data.  One barrier per stage keeps them aligned.
+//
+//  * A: 16-byte global loads, straight into LDS rows (K contiguous).
+//  * B: 16-byte global loads of 8 consecutive columns from 8 consecutive K
+//    rows per thread, an 8 x 8 transpose in registers (v_perm), then one
+//    16-byte LDS write per column.  Sixteen lanes write rows that are 8 apart,
+//    which with a 144-byte pitch would all fall on the same banks; the 16-byte
+//    K blocks of a row are therefore rotated by (row / 16) slots.
+//  * Global loads have two half-stages to land: they are issued right after
+//    the registers they fill were written to LDS, and consumed a full stage
+//    later.  Only LDS traffic is waited for at the barrier.
+template<int64_t BM, int64_t BN, int64_t KC>
+__device__ __forceinline__ void mfma_pingpong(const GlobalView<BM, KC, uint16_t, true> &A,
+                                              const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc<BM, BN, 8> &C) {
+    using Acc = MfmaAcc<BM, BN, 8>;
+    static_assert(BM == 256 && BN == 256, "written for 256 x 256 tiles: 256 movers per operand");
+    constexpr int STAGE_BYTES = (int)(BM + BN) * kMfmaRowBytes;
+    constexpr int TM = Acc::TM, TN = Acc::TN;
+    constexpr int KSTEPS = kMfmaBK / 16;
+
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int group = w / 4;
+    const int t2 = (int)threadIdx.x & 255;
+    const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
+    const int nk = (int)(k_total / kMfmaBK);
+    if (nk == 0) {
+        return;
+    }
+
+    // A movers: chunk t2 % 8 (16 bytes) of rows t2 / 8 + 32 j.
+    const int a_row = t2 / 8, a_kc = t2 % 8;
+    const uint16_t *a_ptr = A.data + (int64_t)a_row * A.lda + a_kc * 8;
+    const int a_step = 32 * (int)A.lda;
+    // B movers: the 8 x 8 block at K block t2 / 32, column block t2 % 32.
+    const int b_nb = t2 % 32, b_kb = t2 / 32;
+    const uint16_t *b_ptr = B.data + (int64_t)(8 * b_kb) * B.lda + 8 * b_nb;
+    const int b_ld = (int)B.lda;
+
+    u32x4_t rr[8];
+    auto fetch = [&](int kt) {
+        const int64_t k0 = (int64_t)kt * kMfmaBK;
+        if (group == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                rr[j] = *reinterpret_cast<const u32x4_t *>(a_ptr + k0 + j * a_step);
+            }
+        } else {
+            const uint16_t *bp = b_ptr + k0 * B.lda;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                rr[j] = *reinterpret_cast<const u32x4_t *>(bp + j * b_ld);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+        if (group == 0) {
+            unsigned char *dst = gern_lds + buf * STAGE_BYTES + a_row * kMfmaRowBytes + a_kc * 16;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                *reinterpret_cast<u32x4_t *>(dst + j * 32 * kMfmaRowBytes) = rr[j];
+            }
+        } else {
+            // rr[r][m] holds columns 2m, 2m+1 of K row r.  Column c of the block
+            // becomes LDS row 8 nb + c, K block kb, in slot (kb + row / 16) % 8.
+            unsigned char *dst = gern_lds + buf * STAGE_BYTES + (int)BM * kMfmaRowBytes + (8 * b_nb) * kMfmaRowBytes +
+                                 ((b_kb + b_nb / 2) & 7) * 16;
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                u32x4_t col;
+                col[0] = __builtin_amdgcn_perm(rr[1][c / 2], rr[0][c / 2], sel);
+                col[1] = __builtin_amdgcn_perm(rr[3][c / 2], rr[2][c / 2], sel);
+                col[2] = __builtin_amdgcn_perm(rr[5][c / 2], rr[4][c / 2], sel);
+                col[3] = __builtin_amdgcn_perm(rr[7][c / 2], rr[6][c / 2], sel);
+                *reinterpret_cast<u32x4_t *>(dst + c * kMfmaRowBytes) = col;
+            }
+        }
+    };
+
+    // Fragment addresses of this lane: row (lane % 32) of each 32-row MFMA
+    // tile, the 16 bytes of K block 2 s + lane / 32 in K step s.
+    const int a_frag = ((w / Acc::WC) * (int)Acc::WM + (lane % 32)) * kMfmaRowBytes + (lane / 32) * 16;
+    const int n0 = (w % Acc::WC) * (int)Acc::WN + (lane % 32);
+    const int b_row0 = (int)BM * kMfmaRowBytes + n0 * kMfmaRowBytes;
+    const int base_slot = (lane / 32) + n0 / 16;
+    int b_off[4];  // slot rotation: K step s of column tile tn sits (s + tn) % 4 double slots on
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        b_off[d] = b_row0 + ((base_slot + 2 * d) & 7) * 16;
+    }
+    auto compute = [&](int kt) {
+        const unsigned char *stage = gern_lds + (kt & 1) * STAGE_BYTES;
+        bf16x8_t af[2][TM], bfr[2][TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) {
+            af[0][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes);
+        }
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) {
+            bfr[0][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_off[tn & 3] + tn * 32 * kMfmaRowBytes);
+        }
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++) {
+            const int cur = s & 1, nxt = cur ^ 1;
+            if (s + 1 < KSTEPS) {
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+                    af[nxt][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + (s + 1) * 32);
+                }
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    bfr[nxt][tn] =
+                        *reinterpret_cast<const bf16x8_t *>(stage + b_off[((s + 1) + tn) & 3] + tn * 32 * kMfmaRowBytes);
+                }
+            }
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+                for (int tn = 0; tn < TN; tn++) {
+                    C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][tm], bfr[cur][tn], C.acc[tm][tn], 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto move = [&](int kt) {
+        if (kt + 1 < nk) {
+            stash((kt + 1) & 1);
+        }
+        if (kt + 2 < nk) {
+            fetch(kt + 2);
+        }
+    };
+    auto lds_barrier = [&]() {
+        // s_waitcnt lgkmcnt(0) with vmcnt and expcnt left at their maxima: the
+        // LDS writes must be done, the global loads stay in flight.
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();
+    };
+
+    fetch(0);
+    stash(0);
+    if (nk > 1) {
+        fetch(1);
+    }
+    lds_barrier();
+    for (int kt = 0; kt < nk; kt++) {
+        if (group == 0) {
+            compute(kt);
+            move(kt);
+        } else {
+            move(kt);
+            compute(kt);
+        }
+        lds_barrier();
+    }
+}
+
+}  // namespace detail
+
 template<int64_t BM, int64_t BN, int64_t KC, int NW, bool EXACT>
 __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t, EXACT> &A,
                                                 const GlobalView<KC, BN, uint16_t, EXACT> &B, MfmaAcc<BM, BN, NW> &C) {
+    if constexpr (NW == 8 && EXACT && BM == 256 && BN == 256) {
+        detail::mfma_pingpong(A, B, C);
+        return;
+    }
     using Acc = MfmaAcc<BM, BN, NW>;
     constexpr int T = Acc::threads;
     static_assert(BM <= 256 && BN <= 256, "tile shape");
