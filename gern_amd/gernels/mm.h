@@ -289,21 +289,22 @@ __device__ __forceinline__ void mfma_pingpong(const GlobalView<BM, KC, uint16_t,
     for (int d = 0; d < 4; d++) {
         b_off[d] = b_row0 + ((base_slot + 2 * d) & 7) * 16;
     }
-    auto compute = [&](int kt) {
+    // K steps [s0, s1) of stage kt, fragments double-buffered in registers.
+    auto compute = [&](int kt, int s0, int s1) {
         const unsigned char *stage = gern_lds + (kt & 1) * STAGE_BYTES;
         bf16x8_t af[2][TM], bfr[2][TN];
 #pragma unroll
         for (int tm = 0; tm < TM; tm++) {
-            af[0][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes);
+            af[s0 & 1][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + s0 * 32);
         }
 #pragma unroll
         for (int tn = 0; tn < TN; tn++) {
-            bfr[0][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_off[tn & 3] + tn * 32 * kMfmaRowBytes);
+            bfr[s0 & 1][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_off[(s0 + tn) & 3] + tn * 32 * kMfmaRowBytes);
         }
 #pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
+        for (int s = s0; s < s1; s++) {
             const int cur = s & 1, nxt = cur ^ 1;
-            if (s + 1 < KSTEPS) {
+            if (s + 1 < s1) {
 #pragma unroll
                 for (int tm = 0; tm < TM; tm++) {
                     af[nxt][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + (s + 1) * 32);
@@ -346,11 +347,14 @@ __device__ __forceinline__ void mfma_pingpong(const GlobalView<BM, KC, uint16_t,
     lds_barrier();
     for (int kt = 0; kt < nk; kt++) {
         if (group == 0) {
-            compute(kt);
+            // Moving in the middle of the stage gives this group's loads a
+            // whole stage to land, like the other group's.
+            compute(kt, 0, KSTEPS / 2);
             move(kt);
+            compute(kt, KSTEPS / 2, KSTEPS);
         } else {
             move(kt);
-            compute(kt);
+            compute(kt, 0, KSTEPS);
         }
         lds_barrier();
     }
