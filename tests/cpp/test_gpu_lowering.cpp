@@ -3,7 +3,8 @@
 // launch dimensions, dynamic LDS with an allocator, LDS-staged tiles.
 //
 // The cases follow the reference's device lowering tests: test/test-gpu-array.cu,
-// test-set-grid.cu, test-dynamic-shared.cu, test-gpu-matrix.cu.
+// test-set-grid.cu, test-dynamic-shared.cu, test-gpu-matrix.cu, and the two
+// reduction programs gernels/cccl/global_reduce.cu and rdom_mimic.cu.
 //
 // With GERN_TEST_COMPILE_ONLY=1 every program is generated and compiled for
 // gfx950 with hiprtc but not loaded or run (no GPU needed).
@@ -18,6 +19,8 @@
 #include "library/array_device_annot.h"
 #include "library/device_host.h"
 #include "library/matrix_device_annot.h"
+
+#include "annot/reduce.h"
 
 #include <cstdlib>
 
@@ -391,6 +394,71 @@ CASE("matrix.add_rows_on_blocks") {
 
 CASE("matrix.add_rows_and_columns_on_blocks") {
     matrix_add(2);
+}
+
+// ---- gernels/cccl: block reduction + device-wide atomic ------------------------------------
+
+CASE("reduce.grid_reduce_total") {  // gernels/cccl/global_reduce.cu:11-66: sum of 0..9 is 45
+    annot::GridReduce grid_reduce;
+    auto input = AbstractDataTypePtr(new const annot::ArrayF32("input"));
+    auto output = AbstractDataTypePtr(new const annot::FloatPtr("output"));
+    Variable block_size{"block_size"}, input_size{"input_size"};
+    const int k_val = 10, threads = 2;
+    input_size = input_size.bind(k_val);
+    auto &specialized = grid_reduce[{{"k", input_size}}];
+    Variable per_block = block_size.bind(threads);
+    Composable program = Global((Reduce(input_size, per_block) || Grid::Unit::BLOCK_X)(specialized(output, input)),
+                                {{Grid::BLOCK_DIM_X, per_block}});
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    impl::ArrayGPU in(k_val), out(1);
+    in.ascending();
+    run.evaluate({{input.getName(), &in}, {output.getName(), &out.data}});
+    REQUIRE_EQ(out.get()[0], (float)(k_val * (k_val - 1) / 2));
+    in.destroy();
+    out.destroy();
+}
+
+static void block_reduce_then_global_sum(int threads, int temp_size_val);
+
+CASE("reduce.block_reduce_whole_wavefronts") {
+    // The same program with 128 threads per block: the sum inside a block is a
+    // wavefront butterfly plus one LDS hop (all partial sums are integers
+    // below 2^24, so the result is exact in any order).
+    block_reduce_then_global_sum(128, 4);
+}
+
+CASE("reduce.block_reduce_then_global_sum") {  // gernels/cccl/rdom_mimic.cu:11-70: sum of 0..7 is 28
+    block_reduce_then_global_sum(2, 4);
+}
+
+static void block_reduce_then_global_sum(int threads, int temp_size_val) {
+    auto input = AbstractDataTypePtr(new const annot::ArrayF32("input"));
+    auto output = AbstractDataTypePtr(new const annot::FloatPtr("output"));
+    auto temp = AbstractDataTypePtr(new const annot::ArrayF32("temp", true));
+    Variable threads_var{"var_thrds_per_blk"}, t1{"t1"}, temp_size("temp_size");
+    Variable bound_threads = threads_var.bind(threads);
+    temp_size = temp_size.bind(temp_size_val);
+    annot::GlobalSum global_sum;
+    annot::BlockReduce block_reduce;
+    auto &block_reduce_sp = block_reduce[{{"block_size", bound_threads}}];
+    (void)global_sum[{{"k", temp_size}}];  // the reference builds this specialisation and calls the plain one
+    Composable program = Global((Reduce(temp_size, t1.bind(1)) || Grid::Unit::BLOCK_X)(block_reduce_sp(temp, input),
+                                                                                         global_sum(output, temp)),
+                                {{Grid::BLOCK_DIM_X, bound_threads}});
+    Runner run(program);
+    if (!build(run, program)) {
+        return;
+    }
+    const int n = temp_size_val * threads;
+    impl::ArrayGPU in(n), out(1);
+    in.ascending();
+    run.evaluate({{input.getName(), &in}, {output.getName(), &out.data}});
+    REQUIRE_EQ(out.get()[0], (float)(n * (n - 1) / 2));
+    in.destroy();
+    out.destroy();
 }
 
 CHECK_MAIN()
