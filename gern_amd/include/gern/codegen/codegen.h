@@ -37,6 +37,9 @@ struct LaunchPlan {
     Expr lds_bytes;                        // undefined = no dynamic LDS
     std::vector<Constraint> host_asserts;  // assumptions checked on the host before each launch
     bool device = false;
+    // Device code that is not a launch: a __device__ function for another
+    // generated kernel to call (FunctionPtr over gernels that occupy grid units).
+    bool device_function = false;
 };
 
 // Values an expression is evaluated against on the host.

@@ -161,6 +161,7 @@ public:
     }
 
     const bool device;
+    bool device_function = false;
     const GeneratorOptions options;
     std::ostringstream body;
     std::set<std::string> headers;
@@ -422,6 +423,10 @@ public:
         Constraint c = substitute(n->constraint, s);
         if (isConstExpr(c)) {
             line(indent, "static_assert(" + gen(c) + ");");
+        } else if (device_function) {
+            // Nobody checks a precondition of a device function that is not a
+            // launch; it is recorded for the reader only.
+            line(indent, "// assumes " + gen(c));
         } else if (!device) {
             line(indent, "assert(" + gen(c) + ");");
         } else {
@@ -439,13 +444,21 @@ public:
 
 std::string CodeGenerator::generate_code(Composable c) {
     const bool device = c.isDeviceLaunch();
+    // A program made of device gernels (its calls occupy grid units) that is
+    // not wrapped in Global() is not launched: it becomes a __device__ function
+    // that another generated kernel calls (FunctionPtr).  The reference only
+    // ever exercised FunctionPtr on the host (test/test-function-ptr.cpp).
+    const bool device_function =
+        !device && c.defined() && getLevel(c.getAnnotation().getOccupiedUnits()) >= Grid::Level::SCALAR;
     NodePtr ir = lower::lowerProgram(c);
 
     Emitter em(device, options);
+    em.device_function = device_function;
     em.emit(ir, 1);
 
     plan = LaunchPlan();
     plan.device = device;
+    plan.device_function = device_function;
     plan.function_name = getUniqueName("function");
 
     plan.grid[0] = em.currentDim(Grid::GRID_DIM_X);
@@ -503,8 +516,8 @@ std::string CodeGenerator::generate_code(Composable c) {
     signature.name = plan.function_name;
     signature.args = parameters;
     signature.template_args = template_args;
-    signature.device = device;
-    signature.access = device ? GLOBAL : HOST;
+    signature.device = device || device_function;
+    signature.access = device ? GLOBAL : (device_function ? DEVICE : HOST);
     signature.grid = LaunchArguments{plan.grid[0], plan.grid[1], plan.grid[2]};
     signature.block = LaunchArguments{plan.block[0], plan.block[1], plan.block[2]};
     signature.smem_size = em.smem_size;
@@ -522,7 +535,7 @@ std::string CodeGenerator::generate_code(Composable c) {
 
     // ---- assemble the file -------------------------------------------------
     std::ostringstream out;
-    if (device) {
+    if (device || device_function) {
         out << "// HIP device code for gfx950, generated by Gern.\n"
                "#if defined(__HIPCC_RTC__)\n"
                "using __hip_internal::int32_t;\n"
@@ -557,6 +570,8 @@ std::string CodeGenerator::generate_code(Composable c) {
             evaluate(plan.block[2], none, bz) && bx * by * bz > 0 && bx * by * bz <= 1024) {
             out << "__launch_bounds__(" << (bx * by * bz) << ") ";
         }
+    } else if (device_function) {
+        out << "__device__ __forceinline__ void ";
     } else {
         out << "void ";
     }
@@ -588,7 +603,7 @@ std::string CodeGenerator::generate_code(Composable c) {
     out << em.body.str();
     out << "}\n";
 
-    if (!device) {
+    if (!device && !device_function) {
         out << "\nextern \"C\" {\nvoid hook_" << plan.function_name << "(void **args) {\n";
         for (const auto &t : template_args) {
             out << "    constexpr int64_t " << t.getName() << " = " << t.getInt64Val() << ";\n";

@@ -64,9 +64,20 @@ void Runner::compile(Options config) {
         out << source;
     }
 
+    if (cg.getLaunchPlan().device_function) {
+        // A __device__ function is only ever #included by another generated
+        // kernel; the file written above is the whole product.
+        if (config.filename.empty()) {
+            throw error::UserError("Runner::Options::filename must be set for a device function: callers include that file");
+        }
+        compiled = false;  // it cannot be evaluated on its own
+        return;
+    }
     if (c.isDeviceLaunch()) {
         plan = std::make_shared<codegen::LaunchPlan>(cg.getLaunchPlan());
         std::vector<std::string> flags = splitIncludeFlags(config.include);
+        // Device functions made by FunctionPtr are written under prefix.
+        flags.push_back("-I" + config.prefix);
         std::vector<const char *> options;
         for (const auto &f : flags) {
             options.push_back(f.c_str());

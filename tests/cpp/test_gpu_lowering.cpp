@@ -396,6 +396,72 @@ CASE("matrix.add_rows_and_columns_on_blocks") {
     matrix_add(2);
 }
 
+// ---- FunctionPtr on the device -----------------------------------------------------------------
+
+static Runner::Options deviceFunctionOptions(const std::string &file) {
+    Runner::Options o;
+    const char *tmp = std::getenv("GERN_TEST_TMP");
+    o.prefix = tmp ? tmp : "/tmp";
+    o.filename = file;
+    o.include = " -I " + libraryDir() + " -I " + packageDir();
+    return o;
+}
+
+// Like build(), with the directory of the device-function files on the include path.
+static bool buildWithPrefix(Runner &run, Composable program, const Runner::Options &inner) {
+    if (compileOnly()) {
+        codegen::CodeGenerator cg;
+        last_source = cg.generate_code(program);
+        const std::string name = cg.getLaunchPlan().name_expression;
+        const std::string i1 = "-I" + libraryDir(), i2 = "-I" + packageDir(), i3 = "-I" + inner.prefix;
+        const char *names[1] = {name.c_str()};
+        const char *opts[3] = {i1.c_str(), i2.c_str(), i3.c_str()};
+        size_t size = 0;
+        if (gern_hip_compile_only(last_source.c_str(), names, 1, opts, 3, "gfx950", &size) != 0) {
+            impl::hipCheck(1);
+        }
+        return false;
+    }
+    Runner::Options o = inner;
+    o.filename = "";
+    run.compile(o);
+    last_source = run.getSource();
+    return true;
+}
+
+CASE("function_ptr.device_function_called_from_a_kernel") {
+    // The host-side cases are test/test-function-ptr.cpp:13-86 of the
+    // reference; here the wrapped program is made of device gernels, so it is
+    // emitted as a __device__ function and called from the generated kernel.
+    auto in = AbstractDataTypePtr(new const annot::ArrayStaticGPU("input_con"));
+    auto temp = AbstractDataTypePtr(new const annot::ArrayStaticGPU("temp", true));
+    auto out = AbstractDataTypePtr(new const annot::ArrayStaticGPU("output_con"));
+    annot::Add1GPUTemplate add_1;
+    Variable step("step"), blk("blk");
+    Runner::Options inner = deviceFunctionOptions("gern_test_device_fn.h");
+    FunctionPtr add_2(Tile(out["size"], step.bind(1))(add_1(in, temp), add_1(temp, out)), inner);
+    REQUIRE(add_2.getFunction().device);
+    // The kernel hands the function views of its arrays (plain ArrayGPU
+    // queries); the function cuts its register arrays out of those.
+    auto in_view = arrayDS("in_view"), out_view = arrayDS("out_view");
+    // (the function's template parameter is bound again where it is called)
+    auto &add_2_bound = add_2[{{"step", step.bind(1)}}];
+    Composable program = Global((Tile(out_view["size"], blk) || Grid::Unit::BLOCK_X)(add_2_bound(in_view, out_view)));
+    Runner run(program);
+    const bool ran = buildWithPrefix(run, program, inner);
+    REQUIRE(last_source.find("gern_test_device_fn.h") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    impl::ArrayGPU a(10), b(10);
+    a.ascending();
+    int64_t blk_val = 5;
+    REQUIRE_NOTHROW(run.evaluate({{in_view.getName(), &a}, {out_view.getName(), &b}, {blk.getName(), &blk_val}}));
+    expect_offset(a, b, 2, 10);
+    a.destroy();
+    b.destroy();
+}
+
 // ---- gernels/cccl: block reduction + device-wide atomic ------------------------------------
 
 CASE("reduce.grid_reduce_total") {  // gernels/cccl/global_reduce.cu:11-66: sum of 0..9 is 45
