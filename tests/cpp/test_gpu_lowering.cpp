@@ -20,6 +20,7 @@
 #include "library/device_host.h"
 #include "library/matrix_device_annot.h"
 
+#include "annot/lds_matrix.h"
 #include "annot/reduce.h"
 
 #include <cstdlib>
@@ -282,14 +283,7 @@ CASE("set_grid.block_size_from_own_variable_and_assumption") {
 
 // ---- test-dynamic-shared.cu ----------------------------------------------------------------
 
-class LdsManager : public grid::SharedMemoryManager {
-public:
-    explicit LdsManager(Variable smem_size)
-        : grid::SharedMemoryManager(
-              FunctionCall{"gernels::lds_init", {smem_size}, {}, Parameter(), LaunchArguments(), LaunchArguments(), DEVICE},
-              {"gernels/lds_alloc.h"}) {
-    }
-};
+using annot::LdsManager;
 
 static void dynamic_lds_run(bool with_manager) {  // test-dynamic-shared.cu:15-105
     auto in = arrayDS("input_con"), out = arrayDS("output_con");
@@ -394,6 +388,77 @@ CASE("matrix.add_rows_on_blocks") {
 
 CASE("matrix.add_rows_and_columns_on_blocks") {
     matrix_add(2);
+}
+
+// ---- user-written GEMM schedule staged through LDS -----------------------------------------------
+
+CASE("schedule.gemm_staged_through_lds") {  // gernels/mm/kernel_3.cu:13-118 of the reference
+    constexpr int64_t m = 128, n = 128, k = 128;
+    using AType = annot::MatrixGlobalToShared<m, k>;
+    using BType = annot::MatrixGlobalToShared<k, n>;
+    using CType = annot::MatrixGlobalToGlobal<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    AType view_of("A_vec", false);
+    Variable k_dim("k_dim"), k_tiled("k_tiled"), block_x("block_x"), block_y("block_y"), thread_x("thread_x"),
+        thread_y("thread_y"), smem_size("smem_size"), one_val("one_val");
+    block_x = block_x.bind(16);
+    block_y = block_y.bind(8);
+    thread_x = thread_x.bind(4);
+    thread_y = thread_y.bind(4);
+    k_dim = k_dim.bind(k);
+    k_tiled = k_tiled.bind(8);
+    one_val = one_val.bind(8);
+    annot::MatrixMultiplyScalar mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    Composable program = Global(
+        (Tile(C["row"], block_x) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y) || Grid::Unit::BLOCK_Y)(Reduce(k_dim, k_tiled)(
+            Stage(A, Stage(B, (Tile(C["row"], thread_x) || Grid::Unit::THREAD_Y)((Tile(C["col"], thread_y) || Grid::Unit::THREAD_X)(
+                                  Reduce(k_dim, one_val)(Stage(A, view_of.getView(), Stage(B, view_of.getView(), mm_sp(A, B, C))))))))))),
+        {}, smem_size, LdsManager(smem_size));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("stage_into_smem") != std::string::npos);
+    REQUIRE(last_source.find("get_view") != std::string::npos);
+    REQUIRE(last_source.find("free_smem") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    impl::MatrixGPU a(m, k, k), b(k, n, n), c(m, n, n);
+    std::vector<float> ha(m * k), hb(k * n);
+    for (int64_t e = 0; e < m * k; e++) {
+        ha[e] = (float)(e % 10);  // the reference's ascending(): i % 10
+    }
+    for (int64_t e = 0; e < k * n; e++) {
+        hb[e] = (float)((e * 7) % 10);
+    }
+    impl::hipCheck(gern_hip_memcpy_h2d(a.data, ha.data(), sizeof(float) * ha.size()));
+    impl::hipCheck(gern_hip_memcpy_h2d(b.data, hb.data(), sizeof(float) * hb.size()));
+    hip::GlobalMatrixF32 pa{a.data}, pb{b.data}, pc{c.data};
+    int64_t smem = 16 * 1024;
+    run.evaluate({{A.getName(), &pa}, {B.getName(), &pb}, {C.getName(), &pc}, {smem_size.getName(), &smem}});
+    std::vector<float> got = c.get();
+    for (int64_t i = 0; i < m; i++) {
+        for (int64_t j = 0; j < n; j++) {
+            float want = 0.0f;
+            for (int64_t kk = 0; kk < k; kk++) {
+                want += ha[i * k + kk] * hb[kk * n + j];
+            }
+            REQUIRE_EQ(got[i * n + j], want);  // small integers: exact in any order
+        }
+    }
+    // a second launch accumulates again: nothing leaked from the LDS allocator
+    run.evaluate({{A.getName(), &pa}, {B.getName(), &pb}, {C.getName(), &pc}, {smem_size.getName(), &smem}});
+    got = c.get();
+    float want00 = 0.0f;
+    for (int64_t kk = 0; kk < k; kk++) {
+        want00 += ha[kk] * hb[kk * n];
+    }
+    REQUIRE_EQ(got[0], 2 * want00);
+    a.destroy();
+    b.destroy();
+    c.destroy();
 }
 
 // ---- FunctionPtr on the device -----------------------------------------------------------------
