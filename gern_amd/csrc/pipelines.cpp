@@ -15,6 +15,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <cstdlib>
 #include <memory>
 #include <string>
 
@@ -71,12 +72,16 @@ int64_t qkWaves(int64_t n) {
 }
 
 // Generates (and, unless compile-only, loads) the program.
-int finish(gern_pipeline_s *p, Composable program, int flags) {
-    const std::string include = "-I " + packageDir();
+int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_simd = 0) {
+    std::string include = "-I " + packageDir();
+    if (const char *extra = std::getenv("GERN_PIPELINE_EXTRA_OPTIONS")) {
+        include += std::string(" ") + extra;  // e.g. "-DNAME=value", for experiments
+    }
     try {
         if (flags & GERN_PIPELINE_COMPILE_ONLY) {
             codegen::GeneratorOptions go;
             go.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+            go.min_waves_per_simd = min_waves_per_simd;
             codegen::CodeGenerator cg(std::nullopt, go);
             p->source = cg.generate_code(program);
             p->kernel_name = cg.getLaunchPlan().name_expression;
@@ -97,6 +102,7 @@ int finish(gern_pipeline_s *p, Composable program, int flags) {
         options.filename = "";  // keep the source in memory only
         options.include = include;
         options.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+        options.min_waves_per_simd = min_waves_per_simd;
         p->runner->compile(options);
         p->source = p->runner->getSource();
         p->names = p->runner->getArgumentOrder();

@@ -27,8 +27,8 @@ constexpr int kLdsMaxBlocks = 14;
 struct LdsTable {
     uint32_t capacity;
     uint32_t count;
-    uint32_t answer;  // the last allocation's offset (0 = none), read by every thread
-    uint32_t pad;
+    uint32_t answer;    // the last allocation's offset, read by every thread
+    uint32_t overflow;  // set once a request could not be met
     uint32_t offset[kLdsMaxBlocks];
     uint32_t size_used[kLdsMaxBlocks];  // size in bytes, bit 0 = in use
 };
@@ -45,14 +45,19 @@ __device__ __forceinline__ void lds_init(int64_t bytes) {
         t->capacity = (uint32_t)bytes;
         t->count = 1;
         t->answer = 0;
+        t->overflow = 0;
         t->offset[0] = first;
         t->size_used[0] = (bytes > first ? ((uint32_t)bytes - first) & ~15u : 0u);
     }
     __syncthreads();
 }
 
-// A 16-byte aligned block of at least `bytes`, or nullptr when nothing fits
-// (or the table is full).
+// A 16-byte aligned block of at least `bytes`.  When nothing fits (or the table
+// is full) the request cannot fail loudly from inside a kernel: the table's
+// overflow flag is set and the START of the heap is returned, so that the
+// caller's accesses stay inside LDS (results are then wrong, as with the
+// reference's allocator once it wraps, but nothing faults).  lds_overflowed()
+// tells.
 __device__ __forceinline__ void *lds_alloc(int64_t bytes) {
     LdsTable *t = reinterpret_cast<LdsTable *>(gern_lds);
     __syncthreads();  // earlier readers of `answer` are done
@@ -80,18 +85,25 @@ __device__ __forceinline__ void *lds_alloc(int64_t bytes) {
             got = t->offset[b];
             break;
         }
+        if (got == 0) {
+            t->overflow = 1;
+            got = (uint32_t)sizeof(LdsTable);
+        }
         t->answer = got;
     }
     __syncthreads();
-    const uint32_t at = t->answer;
-    return at ? gern_lds + at : nullptr;
+    return gern_lds + t->answer;
+}
+
+__device__ __forceinline__ bool lds_overflowed() {
+    return reinterpret_cast<const LdsTable *>(gern_lds)->overflow != 0;
 }
 
 // Returns a block; neighbouring free blocks are merged.
 __device__ __forceinline__ void lds_free(const void *ptr) {
     LdsTable *t = reinterpret_cast<LdsTable *>(gern_lds);
     __syncthreads();  // all readers of the block are done
-    if (lds_first_thread() && ptr != nullptr) {
+    if (lds_first_thread() && ptr != nullptr && !t->overflow) {
         const uint32_t at = (uint32_t)(static_cast<const unsigned char *>(ptr) - gern_lds);
         for (uint32_t b = 0; b < t->count; b++) {
             if (t->offset[b] != at) {

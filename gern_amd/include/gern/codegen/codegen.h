@@ -55,6 +55,9 @@ bool evaluate(const Constraint &c, const EvalEnv &env, bool &value);
 
 struct GeneratorOptions {
     bool xcd_remap = true;
+    // Wavefronts per SIMD the kernel must leave room for (second argument of
+    // __launch_bounds__): caps its registers at 512 / n.  0 = the compiler decides.
+    int min_waves_per_simd = 0;
 };
 
 class CodeGenerator {

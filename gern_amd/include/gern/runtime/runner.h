@@ -42,6 +42,9 @@ public:
         // Spread consecutive workgroups of one XCD over neighbouring tiles
         // (each of the 8 XCDs of an MI355X has its own L2).
         bool xcd_remap = true;
+        // Wavefronts per SIMD the kernel must leave room for (caps its
+        // registers at 512 / n); 0 = the compiler decides.
+        int min_waves_per_simd = 0;
         // HIP stream the kernel is launched on (NULL = default stream).
         void *stream = nullptr;
     };

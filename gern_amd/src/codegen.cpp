@@ -568,7 +568,11 @@ std::string CodeGenerator::generate_code(Composable c) {
         int64_t bx, by, bz;
         if (evaluate(plan.block[0], none, bx) && evaluate(plan.block[1], none, by) &&
             evaluate(plan.block[2], none, bz) && bx * by * bz > 0 && bx * by * bz <= 1024) {
-            out << "__launch_bounds__(" << (bx * by * bz) << ") ";
+            out << "__launch_bounds__(" << (bx * by * bz);
+            if (options.min_waves_per_simd > 0) {
+                out << ", " << options.min_waves_per_simd;
+            }
+            out << ") ";
         }
     } else if (device_function) {
         out << "__device__ __forceinline__ void ";
