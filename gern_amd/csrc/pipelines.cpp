@@ -287,9 +287,13 @@ Composable gemmProgram(annot::MatrixOperand::Element element, bool exact, annot:
     auto C = AbstractDataTypePtr(new const annot::MatrixAccumulator("C", engine, accumulate));
     Variable ti("ti"), tj("tj"), tk("tk"), k_dim("k_dim"), threads("threads"), smem("smem");
     annot::MatrixMultiply mm{A, B, C};
-    return Global((Tile(C["row"], ti.bind(bm)) || Grid::BLOCK_Y)((Tile(C["col"], tj.bind(bn)) || Grid::BLOCK_X)(
-                      Reduce(k_dim, tk.bind(4096))(mm[{{"k_dim", k_dim}}](A, B, C)))),
-                  {{Grid::BLOCK_DIM_X, threads.bind(threads_per_block)}}, smem.bind(lds));
+    Composable tiled = (Tile(C["row"], ti.bind(bm)) || Grid::BLOCK_Y)((Tile(C["col"], tj.bind(bn)) || Grid::BLOCK_X)(
+        Reduce(k_dim, tk.bind(4096))(mm[{{"k_dim", k_dim}}](A, B, C))));
+    if (lds == 0) {
+        // A gernel that keeps its stages in static LDS asks for no dynamic LDS.
+        return Global(tiled, {{Grid::BLOCK_DIM_X, threads.bind(threads_per_block)}});
+    }
+    return Global(tiled, {{Grid::BLOCK_DIM_X, threads.bind(threads_per_block)}}, smem.bind(lds));
 }
 
 }  // namespace
@@ -316,11 +320,12 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                         flags);
             if (rc == 0) {
                 // The same program on data structures that promise whole tiles:
-                // eight wavefronts, no bounds tests.
+                // eight wavefronts, no bounds tests.  That gernel keeps its two
+                // stages in static LDS (gernels/mm.h, mfma_direct): no dynamic LDS.
                 gern_pipeline_s fast;
                 rc = finish(&fast,
                             gemmProgram(annot::MatrixOperand::BF16, true, annot::MatrixAccumulator::MFMA8, accumulate,
-                                        256, 256, 512, lds),
+                                        256, 256, 512, 0),
                             flags);
                 p->exact = std::move(fast.runner);
                 p->exact_source = fast.source;

@@ -194,125 +194,125 @@ namespace detail {
 
 // The fast bf16 path: 256 x 256 tile, eight wavefronts, whole tiles only.
 //
-// Wavefronts 0-3 (one per SIMD) move A, wavefronts 4-7 move B, and the two
-// groups run half a stage out of phase: while one group issues its MFMAs the
-// other writes the next stage into LDS and issues the global loads of the stage
-// after it, so every SIMD always holds one wavefront that computes and one
-// that moves data.  One barrier per stage keeps them aligned.
+// Both operands go from global memory STRAIGHT INTO LDS (global_load_lds, 16
+// bytes per lane, no register round trip, no LDS write instructions), two
+// stages of 64 K each; all eight wavefronts issue the loads of stage k+1,
+// compute stage k, wait for their loads and meet at one barrier.
 //
-//  * A: 16-byte global loads, straight into LDS rows (K contiguous).
-//  * B: 16-byte global loads of 8 consecutive columns from 8 consecutive K
-//    rows per thread, an 8 x 8 transpose in registers (v_perm), then one
-//    16-byte LDS write per column.  Sixteen lanes write rows that are 8 apart,
-//    which with a 144-byte pitch would all fall on the same banks; the 16-byte
-//    K blocks of a row are therefore rotated by (row / 16) slots.
-//  * Global loads have two half-stages to land: they are issued right after
-//    the registers they fill were written to LDS, and consumed a full stage
-//    later.  Only LDS traffic is waited for at the barrier.
+//  * A stage: 256 rows x 128 bytes.  A load instruction fills 1 KiB of LDS in
+//    lane order, so rows cannot be padded; instead the 16-byte chunk c of row
+//    m is kept at position c ^ ((m >> 1) & 7), which spreads the sixteen rows
+//    that one ds_read_b128 pass touches over all 64 banks.  The permutation
+//    is applied on the GLOBAL side (each lane picks the chunk whose home is
+//    its LDS slot) and stays inside 64-byte groups, so loads remain coalesced.
+//  * B stage: 64 K rows x 512 bytes, kept as it lies in memory (columns
+//    contiguous).  The MFMA wants K contiguous per column: ds_read_b64_tr_b16
+//    transposes on the way out (inside each group of sixteen lanes, lane i
+//    receives, as element j, element i % 4 of the 8 bytes addressed by lane
+//    4 j + i / 4).  Chunk c of K row k sits at position c ^ (4 * (k & 3)).
+//  * The two stages are two distinct static arrays: a single dynamic array
+//    would make the compiler wait for the loads into one stage before any
+//    LDS read of the other (it cannot tell them apart), serialising the two.
+//
+// Measured alternatives at 4096^3 (us): register-staged with one barrier per
+// stage 167; two wavefront groups half a stage out of phase (one computing
+// while the other moves data) 140; this one 129-133.
 template<int64_t BM, int64_t BN, int64_t KC>
-__device__ __forceinline__ void mfma_pingpong(const GlobalView<BM, KC, uint16_t, true> &A,
-                                              const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc<BM, BN, 8> &C) {
+__device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, true> &A,
+                                            const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc<BM, BN, 8> &C) {
     using Acc = MfmaAcc<BM, BN, 8>;
-    static_assert(BM == 256 && BN == 256, "written for 256 x 256 tiles: 256 movers per operand");
-    constexpr int STAGE_BYTES = (int)(BM + BN) * kMfmaRowBytes;
+    static_assert(BM == 256 && BN == 256, "written for 256 x 256 tiles");
     constexpr int TM = Acc::TM, TN = Acc::TN;
     constexpr int KSTEPS = kMfmaBK / 16;
+    constexpr int A_BYTES = 256 * 128;
+    constexpr int STAGE = A_BYTES + 64 * 512;
+    typedef short v4s_t __attribute__((ext_vector_type(4)));
+    typedef short v8s_t __attribute__((ext_vector_type(8)));
+    __shared__ __attribute__((aligned(16))) unsigned char stage_even[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char stage_odd[STAGE];
 
     const int lane = lane_id();
     const int w = wave_in_block();
-    const int group = w / 4;
-    const int t2 = (int)threadIdx.x & 255;
     const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
     const int nk = (int)(k_total / kMfmaBK);
     if (nk == 0) {
         return;
     }
 
-    // A movers: chunk t2 % 8 (16 bytes) of rows t2 / 8 + 32 j.
-    const int a_row = t2 / 8, a_kc = t2 % 8;
-    const uint16_t *a_ptr = A.data + (int64_t)a_row * A.lda + a_kc * 8;
-    const int a_step = 32 * (int)A.lda;
-    // B movers: the 8 x 8 block at K block t2 / 32, column block t2 % 32.
-    const int b_nb = t2 % 32, b_kb = t2 / 32;
-    const uint16_t *b_ptr = B.data + (int64_t)(8 * b_kb) * B.lda + 8 * b_nb;
-    const int b_ld = (int)B.lda;
-
-    u32x4_t rr[8];
-    auto fetch = [&](int kt) {
+    // Wavefront w issues A instructions 4w .. 4w+3 (8 rows each) and B
+    // instructions 4w .. 4w+3 (2 K rows each) of every stage.
+    auto issue = [&](int kt, unsigned char *dst) {
         const int64_t k0 = (int64_t)kt * kMfmaBK;
-        if (group == 0) {
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                rr[j] = *reinterpret_cast<const u32x4_t *>(a_ptr + k0 + j * a_step);
-            }
-        } else {
-            const uint16_t *bp = b_ptr + k0 * B.lda;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                rr[j] = *reinterpret_cast<const u32x4_t *>(bp + j * b_ld);
-            }
+        for (int j = 0; j < 4; j++) {
+            const int i = w * 4 + j;
+            const int row = 8 * i + lane / 8;
+            const int c = (lane % 8) ^ ((row >> 1) & 7);
+            const uint16_t *src = A.data + k0 + (uint32_t)(row * (int)A.lda + c * 8);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16, 0, 0);
         }
-    };
-    auto stash = [&](int buf) {
-        if (group == 0) {
-            unsigned char *dst = gern_lds + buf * STAGE_BYTES + a_row * kMfmaRowBytes + a_kc * 16;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                *reinterpret_cast<u32x4_t *>(dst + j * 32 * kMfmaRowBytes) = rr[j];
-            }
-        } else {
-            // rr[r][m] holds columns 2m, 2m+1 of K row r.  Column c of the block
-            // becomes LDS row 8 nb + c, K block kb, in slot (kb + row / 16) % 8.
-            unsigned char *dst = gern_lds + buf * STAGE_BYTES + (int)BM * kMfmaRowBytes + (8 * b_nb) * kMfmaRowBytes +
-                                 ((b_kb + b_nb / 2) & 7) * 16;
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                u32x4_t col;
-                col[0] = __builtin_amdgcn_perm(rr[1][c / 2], rr[0][c / 2], sel);
-                col[1] = __builtin_amdgcn_perm(rr[3][c / 2], rr[2][c / 2], sel);
-                col[2] = __builtin_amdgcn_perm(rr[5][c / 2], rr[4][c / 2], sel);
-                col[3] = __builtin_amdgcn_perm(rr[7][c / 2], rr[6][c / 2], sel);
-                *reinterpret_cast<u32x4_t *>(dst + c * kMfmaRowBytes) = col;
-            }
+        for (int j = 0; j < 4; j++) {
+            const int i = w * 4 + j;
+            const int krow = 2 * i + lane / 32;
+            const int c = (lane % 32) ^ (4 * (krow & 3));
+            const uint16_t *src = B.data + k0 * B.lda + (uint32_t)(krow * (int)B.lda + c * 8);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)), 16, 0, 0);
         }
     };
 
-    // Fragment addresses of this lane: row (lane % 32) of each 32-row MFMA
-    // tile, the 16 bytes of K block 2 s + lane / 32 in K step s.
-    const int a_frag = ((w / Acc::WC) * (int)Acc::WM + (lane % 32)) * kMfmaRowBytes + (lane / 32) * 16;
-    const int n0 = (w % Acc::WC) * (int)Acc::WN + (lane % 32);
-    const int b_row0 = (int)BM * kMfmaRowBytes + n0 * kMfmaRowBytes;
-    const int base_slot = (lane / 32) + n0 / 16;
-    int b_off[4];  // slot rotation: K step s of column tile tn sits (s + tn) % 4 double slots on
-#pragma unroll
-    for (int d = 0; d < 4; d++) {
-        b_off[d] = b_row0 + ((base_slot + 2 * d) & 7) * 16;
-    }
-    // K steps [s0, s1) of stage kt, fragments double-buffered in registers.
-    auto compute = [&](int kt, int s0, int s1) {
-        const unsigned char *stage = gern_lds + (kt & 1) * STAGE_BYTES;
+    // A fragment of this lane: row lane % 32 of each 32-row tile, K block
+    // 2 s + lane / 32 of K step s.
+    const int a_row_off = ((w / Acc::WC) * (int)Acc::WM + (lane % 32)) * 128;
+    const int a_swz = ((lane % 32) >> 1) & 7;
+    const int a_half = lane / 32;
+    // B fragment: lane p of 16-lane group g addresses K row 16 s + 8 (g / 2) +
+    // 4 q + p / 4, columns 16 (g % 2) + 4 (p % 4) .. + 3 of the 32-column tile;
+    // the transposing read hands it K rows 8 (g / 2) + 4 q .. + 3 of column
+    // 16 (g % 2) + p, which is what MFMA lane 16 g + p holds.
+    const int g = lane / 16, p = lane % 16;
+    const int b_col0 = (w % Acc::WC) * (int)Acc::WN + 16 * (g % 2);
+    const int b_krow = 8 * (g / 2) + p / 4;
+    const int b_swz = 4 * (p / 4);  // (k & 3) == p / 4: the other terms are multiples of 4
+    // Every LDS address below is ONE offset from the stage array: the compiler
+    // tells the two stages apart only through short pointer chains.
+    auto load_a = [&](const unsigned char *stage, int tm, int s) {
+        const int pos = (2 * s + a_half) ^ a_swz;
+        const int at = a_row_off + tm * 32 * 128 + pos * 16;
+        return *reinterpret_cast<const bf16x8_t *>(stage + at);
+    };
+    auto load_b = [&](const unsigned char *stage, int tn, int s) {
+        const int chunk = ((b_col0 + tn * 32) / 8 + (p % 4) / 2) ^ b_swz;
+        const int at = A_BYTES + (16 * s + b_krow) * 512 + chunk * 16 + (p % 2) * 8;
+        const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + at));
+        const v4s_t hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + (at + 4 * 512)));
+        const v8s_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return __builtin_bit_cast(bf16x8_t, both);
+    };
+    auto compute = [&](const unsigned char *stage) {
         bf16x8_t af[2][TM], bfr[2][TN];
 #pragma unroll
         for (int tm = 0; tm < TM; tm++) {
-            af[s0 & 1][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + s0 * 32);
+            af[0][tm] = load_a(stage, tm, 0);
         }
 #pragma unroll
         for (int tn = 0; tn < TN; tn++) {
-            bfr[s0 & 1][tn] = *reinterpret_cast<const bf16x8_t *>(stage + b_off[(s0 + tn) & 3] + tn * 32 * kMfmaRowBytes);
+            bfr[0][tn] = load_b(stage, tn, 0);
         }
 #pragma unroll
-        for (int s = s0; s < s1; s++) {
+        for (int s = 0; s < KSTEPS; s++) {
             const int cur = s & 1, nxt = cur ^ 1;
-            if (s + 1 < s1) {
+            if (s + 1 < KSTEPS) {
 #pragma unroll
                 for (int tm = 0; tm < TM; tm++) {
-                    af[nxt][tm] = *reinterpret_cast<const bf16x8_t *>(stage + a_frag + tm * 32 * kMfmaRowBytes + (s + 1) * 32);
+                    af[nxt][tm] = load_a(stage, tm, s + 1);
                 }
 #pragma unroll
                 for (int tn = 0; tn < TN; tn++) {
-                    bfr[nxt][tn] =
-                        *reinterpret_cast<const bf16x8_t *>(stage + b_off[((s + 1) + tn) & 3] + tn * 32 * kMfmaRowBytes);
+                    bfr[nxt][tn] = load_b(stage, tn, s + 1);
                 }
             }
 #pragma unroll
@@ -324,39 +324,28 @@ __device__ __forceinline__ void mfma_pingpong(const GlobalView<BM, KC, uint16_t,
             }
         }
     };
-    auto move = [&](int kt) {
-        if (kt + 1 < nk) {
-            stash((kt + 1) & 1);
-        }
-        if (kt + 2 < nk) {
-            fetch(kt + 2);
-        }
-    };
-    auto lds_barrier = [&]() {
-        // s_waitcnt lgkmcnt(0) with vmcnt and expcnt left at their maxima: the
-        // LDS writes must be done, the global loads stay in flight.
-        __builtin_amdgcn_s_waitcnt(0xC07F);
+    auto arrive = [&]() {
+        // vmcnt(0) lgkmcnt(0): this wavefront's loads have landed in LDS and its
+        // LDS reads are done; then everybody's.
+        __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
     };
 
-    fetch(0);
-    stash(0);
-    if (nk > 1) {
-        fetch(1);
-    }
-    lds_barrier();
-    for (int kt = 0; kt < nk; kt++) {
-        if (group == 0) {
-            // Moving in the middle of the stage gives this group's loads a
-            // whole stage to land, like the other group's.
-            compute(kt, 0, KSTEPS / 2);
-            move(kt);
-            compute(kt, KSTEPS / 2, KSTEPS);
-        } else {
-            move(kt);
-            compute(kt, 0, KSTEPS);
+    issue(0, stage_even);
+    arrive();
+    for (int kt = 0; kt < nk; kt += 2) {
+        if (kt + 1 < nk) {
+            issue(kt + 1, stage_odd);
         }
-        lds_barrier();
+        compute(stage_even);
+        arrive();
+        if (kt + 1 < nk) {
+            if (kt + 2 < nk) {
+                issue(kt + 2, stage_even);
+            }
+            compute(stage_odd);
+            arrive();
+        }
     }
 }
 
@@ -366,7 +355,7 @@ template<int64_t BM, int64_t BN, int64_t KC, int NW, bool EXACT>
 __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t, EXACT> &A,
                                                 const GlobalView<KC, BN, uint16_t, EXACT> &B, MfmaAcc<BM, BN, NW> &C) {
     if constexpr (NW == 8 && EXACT && BM == 256 && BN == 256) {
-        detail::mfma_pingpong(A, B, C);
+        detail::mfma_direct(A, B, C);
         return;
     }
     using Acc = MfmaAcc<BM, BN, NW>;

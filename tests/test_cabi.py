@@ -132,3 +132,33 @@ def test_headline_kernels_use_no_scratch_memory(tmp_path, name, make):
     for k in _kernel_notes(tmp_path, make):
         assert k[".vgpr_spill_count"] == 0, (name, k)
         assert k[".private_segment_fixed_size"] == 0, (name, k)
+
+
+def test_bf16_gemm_reads_one_stage_while_the_other_fills(tmp_path):
+    # The whole-tile bf16 GEMM loads stage k+1 straight into LDS while it reads
+    # stage k.  The compiler keeps the two apart only while every LDS address is
+    # a short pointer chain from its own static array; when it loses track it
+    # waits for all outstanding loads (a bare "s_waitcnt vmcnt(0)") before the
+    # first LDS read, which serialises fetch and compute (measured: +8 %).
+    import shutil
+    import subprocess
+    objdump = shutil.which("llvm-objdump") or "/opt/rocm/llvm/bin/llvm-objdump"
+    if not os.path.exists(objdump):
+        pytest.skip("llvm-objdump not available")
+    os.environ["GERN_HIP_KEEP_DIR"] = str(tmp_path)
+    try:
+        gern_amd.Gemm("bf16", overwrite=True, flags=gern_amd.COMPILE_ONLY)
+    finally:
+        del os.environ["GERN_HIP_KEEP_DIR"]
+    checked = 0
+    for f in sorted(tmp_path.glob("*.hsaco")):
+        text = subprocess.run([objdump, "-d", str(f)], stdout=subprocess.PIPE, text=True, check=True).stdout
+        if "global_load_lds_dwordx4" not in text:
+            continue  # the general (ragged) kernel stages through registers
+        checked += 1
+        lines = [l.split("//")[0].strip() for l in text.splitlines()]
+        first = next(i for i, l in enumerate(lines) if l.startswith("global_load_lds"))
+        last = max(i for i, l in enumerate(lines) if l.startswith("v_mfma"))
+        bare = [l for l in lines[first:last] if l.startswith("s_waitcnt") and "vmcnt(0)" in l and "lgkmcnt" not in l]
+        assert not bare, bare
+    assert checked == 1
