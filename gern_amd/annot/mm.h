@@ -138,7 +138,11 @@ public:
                                                                  SubsetObj(B, {k, j, tk, tj}),
                                                              })))))
             // all threads of a workgroup cooperate
-            .occupies({Grid::Unit::THREAD_X});
+            .occupies({Grid::Unit::THREAD_X})
+            // the whole-tile bf16 gernel addresses a tile with 32-bit byte
+            // offsets (gernels/mm.h, kMfmaMaxLd)
+            .assumes(Constraint(ADTMember(A, "lda", false) <= Expr((int64_t)1 << 21)),
+                     Constraint(ADTMember(B, "lda", false) <= Expr((int64_t)1 << 21)));
     }
     FunctionSignature getFunction() override {
         FunctionSignature f;

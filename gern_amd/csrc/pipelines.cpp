@@ -372,7 +372,9 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    p->last_run_exact = p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0;
+    // whole tiles, and row pitches (K for A, N for B) within the fast gernel's 32-bit byte offsets
+    p->last_run_exact =
+        p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K <= (int64_t(1) << 21) && N <= (int64_t(1) << 21);
     if (p->last_run_exact) {
         runner = p->exact.get();
     }

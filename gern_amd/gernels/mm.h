@@ -182,6 +182,7 @@ __device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const
 }
 
 constexpr int kMfmaBK = 64;                      // K depth of one LDS stage
+constexpr int64_t kMfmaMaxLd = 1 << 21;          // whole-tile bf16 path: row pitch of A and B, in elements
 constexpr int kMfmaRowBytes = 2 * kMfmaBK + 16;  // padded LDS row: 144 bytes
 
 // LDS needed by matrix_multiply on bf16 operands.
@@ -194,7 +195,7 @@ namespace detail {
 
 // The fast bf16 path: 256 x 256 tile, eight wavefronts, whole tiles only.
 //
-// Both operands go from global memory STRAIGHT INTO LDS (global_load_lds, 16
+// Both operands go from global memory STRAIGHT INTO LDS (buffer_load ... lds, 16
 // bytes per lane, no register round trip, no LDS write instructions), two
 // stages of 64 K each; all eight wavefronts issue the loads of stage k+1,
 // compute stage k, wait for their loads and meet at one barrier.
@@ -240,26 +241,44 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     }
 
     // Wavefront w issues A instructions 4w .. 4w+3 (8 rows each) and B
-    // instructions 4w .. 4w+3 (2 K rows each) of every stage.
+    // instructions 4w .. 4w+3 (2 K rows each) of every stage, as buffer loads:
+    // descriptor and per-instruction byte offset live in scalar registers, the
+    // lane's own offset is one of two constants (it depends on the parity of
+    // the instruction only), so issuing a stage takes no vector ALU work.  It
+    // matters: the SIMD hands its vector-ALU slot to the oldest wavefront, and
+    // one that streams MFMAs starves the address arithmetic of the other
+    // (64-bit lane addresses made this kernel 10 % slower).
+    // Byte offsets are 32 bit: lda and ldb below kMfmaMaxLd elements.
+    const int wu = __builtin_amdgcn_readfirstlane(w);
+    int lane_off_a[2], lane_off_b[2];
+#pragma unroll
+    for (int odd = 0; odd < 2; odd++) {
+        // A: row 8 i + lane / 8, chunk (lane % 8) ^ ((row >> 1) & 7); B: K row
+        // 2 i + lane / 32, chunk (lane % 32) ^ (4 * (K row & 3)); i = 4 w + j
+        const int chunk_a = (lane % 8) ^ ((4 * odd + lane / 16) & 7);
+        lane_off_a[odd] = ((lane / 8) * (int)A.lda + chunk_a * 8) * 2;
+        const int chunk_b = (lane % 32) ^ (4 * ((2 * odd + lane / 32) & 3));
+        lane_off_b[odd] = ((lane / 32) * (int)B.lda + chunk_b * 8) * 2;
+    }
+    constexpr int kRawBuffer = 0x00020000;  // 32-bit raw buffer descriptor, no swizzle, no bounds beyond num_records
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, -1, kRawBuffer);
+    const int row_bytes_a = (int)A.lda * 2, row_bytes_b = (int)B.lda * 2;
     auto issue = [&](int kt, unsigned char *dst) {
-        const int64_t k0 = (int64_t)kt * kMfmaBK;
+        const int k0 = kt * (int)kMfmaBK;
+        const __amdgpu_buffer_rsrc_t desc_b =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(B.data + (int64_t)k0 * B.lda), 0, -1, kRawBuffer);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int i = w * 4 + j;
-            const int row = 8 * i + lane / 8;
-            const int c = (lane % 8) ^ ((row >> 1) & 7);
-            const uint16_t *src = A.data + k0 + (uint32_t)(row * (int)A.lda + c * 8);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                             (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16, 0, 0);
+            const int i = wu * 4 + j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
+                                                     lane_off_a[j & 1], k0 * 2 + 8 * i * row_bytes_a, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int i = w * 4 + j;
-            const int krow = 2 * i + lane / 32;
-            const int c = (lane % 32) ^ (4 * (krow & 3));
-            const uint16_t *src = B.data + k0 * B.lda + (uint32_t)(krow * (int)B.lda + c * 8);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                             (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)), 16, 0, 0);
+            const int i = wu * 4 + j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b,
+                                                     (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)),
+                                                     16, lane_off_b[j & 1], 2 * i * row_bytes_b, 0, 0);
         }
     };
 

@@ -153,11 +153,12 @@ def test_bf16_gemm_reads_one_stage_while_the_other_fills(tmp_path):
     checked = 0
     for f in sorted(tmp_path.glob("*.hsaco")):
         text = subprocess.run([objdump, "-d", str(f)], stdout=subprocess.PIPE, text=True, check=True).stdout
-        if "global_load_lds_dwordx4" not in text:
+        lines = [l.split("//")[0].strip() for l in text.splitlines()]
+        to_lds = [i for i, l in enumerate(lines) if l.startswith("buffer_load_dwordx4") and l.endswith(" lds")]
+        if not to_lds:
             continue  # the general (ragged) kernel stages through registers
         checked += 1
-        lines = [l.split("//")[0].strip() for l in text.splitlines()]
-        first = next(i for i, l in enumerate(lines) if l.startswith("global_load_lds"))
+        first = to_lds[0]
         last = max(i for i, l in enumerate(lines) if l.startswith("v_mfma"))
         bare = [l for l in lines[first:last] if l.startswith("s_waitcnt") and "vmcnt(0)" in l and "lgkmcnt" not in l]
         assert not bare, bare
