@@ -116,6 +116,98 @@ __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y,
     }
 }
 
+namespace detail {
+
+// Q K^T of one wavefront's columns with K streamed through LDS, for head
+// dimensions whose rows fill whole load instructions (D = 32, 64, 128, 256).
+//
+// A tile is the 16 keys of one MFMA (keys 4 j + t of a 64-key group, see
+// RowBlock) x D: 32 D bytes.  It is fetched with loads that write straight
+// into LDS (16 bytes per lane, lanes in LDS order): sixteen-byte piece `slot`
+// of key j lands at j * 2 D + slot * 16, and holds piece slot ^ swz(j) of the
+// key, so that the sixteen lanes of one LDS read pass (sixteen keys, the same
+// piece) fall into sixteen different 16-byte bank groups.  Consecutive lanes
+// read consecutive bytes of one key: whole cache lines per lane group, and no
+// cross-lane shuffle afterwards (loading in the MFMA's own lane order costs
+// four ds_bpermute per load).  Each wavefront owns its keys, so the pipeline
+// is private to the wavefront (P tiles in flight, no workgroup barrier); the
+// P slots are separate arrays for the compiler to order loads and reads per
+// slot instead of waiting for every outstanding load.
+template<int64_t R, int64_t N, int64_t D>
+__device__ __forceinline__ void qk_through_lds(const bf16x8_t (&q)[D / 32], const GlobalView<N, D, uint16_t, false> &K,
+                                               RowBlock<R, N> &S, float to_log2) {
+    using Block = RowBlock<R, N>;
+    constexpr int NW = Block::NW;
+    constexpr int KS = (int)(D / 32);
+    constexpr int PR = (int)(D / 8);            // 16-byte pieces per key
+    constexpr int TILE = 32 * (int)D;           // bytes of a tile
+    constexpr int LOADS = TILE / 1024;          // load instructions per tile
+    constexpr int KEYS_PER_LOAD = 16 / LOADS;
+    constexpr int P = TILE >= 8192 ? 2 : 4;     // tiles in flight (at most 16 KiB per wavefront)
+    constexpr int TILES = Block::G * 4;
+    static_assert(TILE % 1024 == 0 && 64 % PR == 0 || PR == 32, "rows fill whole load instructions");
+    __shared__ __attribute__((aligned(16))) unsigned char k_slot0[NW * TILE];
+    __shared__ __attribute__((aligned(16))) unsigned char k_slot1[NW * TILE];
+    __shared__ __attribute__((aligned(16))) unsigned char k_slot2[P == 4 ? NW * TILE : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char k_slot3[P == 4 ? NW * TILE : 16];
+
+    const int lane = lane_id();
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
+    // swz(j): what the piece index of key j is XORed with
+    auto swz = [](int j) { return PR >= 16 ? j % 16 : (j / (16 / PR)) % PR; };
+    const int last_key = (int)K.rows - 1;
+    const int row_bytes = (int)K.lda * 2;
+    constexpr int kRawBuffer = 0x00020000;
+    // no key at all: a descriptor of zero bytes makes every load return zeros without touching memory
+    const __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc((void *)K.data, 0, last_key >= 0 ? -1 : 0, kRawBuffer);
+    const int wave_key0 = w * (int)Block::wave_cols;
+
+    auto slot_of = [&](int tile) -> unsigned char * {
+        switch (tile % P) {
+        case 0: return k_slot0;
+        case 1: return k_slot1;
+        case 2: return k_slot2;
+        default: return k_slot3;
+        }
+    };
+    auto issue = [&](int tile) {
+        const int g = tile / 4, t = tile % 4;
+        unsigned char *dst = slot_of(tile);
+#pragma unroll
+        for (int i = 0; i < LOADS; i++) {
+            const int j = i * KEYS_PER_LOAD + lane / PR;
+            const int piece = (lane % PR) ^ swz(j);
+            int key = wave_key0 + 64 * g + 4 * j + t;
+            key = key < last_key ? key : last_key;  // keys past the end are masked below; read a valid one
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc, (__attribute__((address_space(3))) void *)(dst + (w * TILE + i * 1024)),
+                                                     16, key * row_bytes + piece * 16, 0, 0, 0);
+        }
+    };
+    const int j_mine = lane % 16;
+    const int frag_base = w * TILE + j_mine * 2 * (int)D;
+#pragma unroll
+    for (int tile = 0; tile < P - 1 && tile < TILES; tile++) {
+        issue(tile);
+    }
+#pragma unroll
+    for (int tile = 0; tile < TILES; tile++) {
+        if (tile + P - 1 < TILES) {
+            issue(tile + P - 1);
+        }
+        const unsigned char *src = slot_of(tile);
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const int slot = (4 * s + lane / 16) ^ swz(j_mine);
+            const bf16x8_t k = *reinterpret_cast<const bf16x8_t *>(src + (frag_base + slot * 16));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(q[s], k, acc, 0, 0, 0);
+        }
+        S.acc[tile / 4][tile % 4] = acc * to_log2;
+    }
+}
+
+}  // namespace detail
+
 // S = log2(e) * scale * Q K^T for the 16 rows of Q in view (log2 units, see
 // exp_matrix below); columns past the last key get -inf so that they vanish
 // from the softmax.
@@ -140,6 +232,13 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
             q[s] = __builtin_bit_cast(bf16x8_t, v);
         }
     }
+    // The logits are kept in log2 units (scale * log2(e) folded into one
+    // multiply), so that the exp stage is a bare v_exp_f32.
+    const float to_log2 = scale * 1.4426950408889634f;
+    if constexpr (D == 32 || D == 64 || D == 128 || D == 256) {
+        detail::qk_through_lds<R, N, D>(q, K, S, to_log2);
+    } else {
+    // Other head dimensions: K goes through registers.
     // K is read with lanes 4j .. 4j+3 on the four 16-byte pieces of ONE key's
     // 64 bytes (sixteen keys per load), so that each group of four lanes
     // touches a single cache line: the vector cache looks up one line per
@@ -148,9 +247,6 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
     // The pieces then move to the lanes that feed the MFMA with ds_bpermute
     // (lane l takes from lane 4*(l%16) + l/16), which costs no LDS space.
     const int take_from = 4 * (4 * (lane % 16) + lane / 16);
-    // The logits are kept in log2 units (scale * log2(e) folded into one
-    // multiply), so that the exp stage is a bare v_exp_f32.
-    const float to_log2 = scale * 1.4426950408889634f;
 #pragma unroll
     for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
@@ -172,8 +268,12 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
             }
             S.acc[g][t] = acc * to_log2;
         }
-        // The column a lane holds in tile t is its own key, so validity is a
-        // per-lane, per-tile property.
+    }
+    }
+    // The column a lane holds in tile t is its own key, so validity is a
+    // per-lane, per-tile property.
+#pragma unroll
+    for (int g = 0; g < RowBlock<R, N>::G; g++) {
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             const int64_t key = (int64_t)w * RowBlock<R, N>::wave_cols + 64 * g + 4 * (lane % 16) + t;

@@ -245,8 +245,11 @@ def _run_qk(gpu, qb, kb, scale, max_keys):
     return S.cpu().numpy()
 
 
+# head dimensions 32, 64, 128 and 256 stream K through LDS (256: two tiles in
+# flight instead of four), 96 takes the register path; ragged rows and keys
 @pytest.mark.parametrize("M,N,D,max_keys", [(64, 256, 128, 256), (50, 200, 64, 256), (16, 1024, 128, 1024),
-                                            (37, 1000, 32, 1024)])
+                                            (37, 1000, 32, 1024), (33, 500, 256, 512), (20, 300, 96, 512),
+                                            (48, 2048, 256, 2048)])
 def test_qk_softmax_matches_oracle(gpu, oracle, M, N, D, max_keys):
     qb, _ = oracle.to_bf16(oracle.normal((M, D), 5))
     kb, _ = oracle.to_bf16(oracle.normal((N, D), 6))
