@@ -189,6 +189,39 @@ def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K):
     assert np.array_equal(_run_gemm(gpu, "bf16", aib, bib), ai @ bi)
 
 
+# Shapes made of whole 256 x 256 tiles take the eight-wavefront kernel that
+# loads straight into LDS: one K stage, an odd number of stages, several
+# column and row tiles, and a K that spans more than one 4096-deep Reduce step.
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 768, 128), (768, 512, 4096 + 4096 + 64)])
+@pytest.mark.parametrize("overwrite", [False, True])
+def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
+    import torch
+    # small integers: every product and every partial sum is exact in fp32 in
+    # any order, so each element of C pins its own row of A and column of B
+    ai = np.random.RandomState(11).randint(-3, 4, size=(M, K)).astype(np.float32)
+    bi = np.random.RandomState(12).randint(-3, 4, size=(K, N)).astype(np.float32)
+    c0 = np.random.RandomState(13).randint(-5, 6, size=(M, N)).astype(np.float32)
+    aib, _ = oracle.to_bf16(ai)
+    bib, _ = oracle.to_bf16(bi)
+    g = gpu.Gemm("bf16", overwrite=overwrite)
+    dC = _dev(c0)
+    g(_dev(aib.view(np.int16)), _dev(bib.view(np.int16)), dC)
+    torch.cuda.synchronize()
+    assert "256, 256" in g.kernel_name and "512" in g.kernel_name.split("<")[1].split(",")[0], g.kernel_name
+    want = ai.astype(np.float64) @ bi.astype(np.float64) + (0 if overwrite else c0)
+    assert np.array_equal(dC.cpu().numpy().astype(np.float64), want)
+    # and ordinary values against the oracle
+    ab, _ = oracle.to_bf16(oracle.uniform((M, K), 21, -1.0, 1.0))
+    bb, _ = oracle.to_bf16(oracle.uniform((K, N), 22, -1.0, 1.0))
+    dC = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    g(_dev(ab.view(np.int16)), _dev(bb.view(np.int16)), dC)
+    torch.cuda.synchronize()
+    rows = (M - 2, M)
+    want = oracle.gemm_bf16(ab, bb, rows=rows)[rows[0]:rows[1]]
+    got = dC.cpu().numpy()[rows[0]:rows[1]]
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
+
+
 @pytest.mark.parametrize("variant", ["f32", "bf16"])
 def test_gemm_accumulates_into_c(gpu, oracle, variant):
     A = oracle.uniform((192, 128), 3, -1.0, 1.0)
