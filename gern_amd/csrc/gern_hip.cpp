@@ -36,40 +36,44 @@ int hip_fail(hipError_t e, const char *what) {
         }                                       \
     } while (0)
 
+// Limits of each device, read once per device: launches are checked against
+// the limits of the device that is current in the calling thread.
 std::mutex g_limits_mutex;
-bool g_limits_ready = false;
-gern_hip_limits g_limits;
+std::map<int, gern_hip_limits> g_limits_by_device;
 
-int load_limits() {
-    std::lock_guard<std::mutex> lock(g_limits_mutex);
-    if (g_limits_ready) {
-        return GERN_HIP_OK;
-    }
-    int count = 0;
-    hipError_t e = hipGetDeviceCount(&count);
-    if (e != hipSuccess || count == 0) {
+int current_limits(gern_hip_limits &out) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) {
         return fail(GERN_HIP_ERR_NO_DEVICE, "no HIP device is visible to this process");
     }
+    std::lock_guard<std::mutex> lock(g_limits_mutex);
+    auto it = g_limits_by_device.find(device);
+    if (it != g_limits_by_device.end()) {
+        out = it->second;
+        return GERN_HIP_OK;
+    }
     hipDeviceProp_t prop;
-    HIP_TRY(hipGetDeviceProperties(&prop, 0));
-    std::memset(&g_limits, 0, sizeof(g_limits));
-    g_limits.wavefront_size = prop.warpSize;
-    g_limits.max_threads_per_block = prop.maxThreadsPerBlock;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    gern_hip_limits limits;
+    std::memset(&limits, 0, sizeof(limits));
+    limits.wavefront_size = prop.warpSize;
+    limits.max_threads_per_block = prop.maxThreadsPerBlock;
     for (int i = 0; i < 3; i++) {
-        g_limits.max_block_dim[i] = prop.maxThreadsDim[i];
-        g_limits.max_grid_dim[i] = prop.maxGridSize[i];
+        limits.max_block_dim[i] = prop.maxThreadsDim[i];
+        limits.max_grid_dim[i] = prop.maxGridSize[i];
     }
-    g_limits.lds_bytes_per_block = (int64_t)prop.sharedMemPerBlock;
+    limits.lds_bytes_per_block = (int64_t)prop.sharedMemPerBlock;
     int optin = 0;
-    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, 0) == hipSuccess &&
-        optin > g_limits.lds_bytes_per_block) {
-        g_limits.lds_bytes_per_block = optin;
+    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, device) == hipSuccess &&
+        optin > limits.lds_bytes_per_block) {
+        limits.lds_bytes_per_block = optin;
     }
-    g_limits.compute_units = prop.multiProcessorCount;
-    g_limits.clock_khz = prop.clockRate;
-    g_limits.hbm_bytes = (int64_t)prop.totalGlobalMem;
-    std::snprintf(g_limits.arch, sizeof(g_limits.arch), "%s", prop.gcnArchName);
-    g_limits_ready = true;
+    limits.compute_units = prop.multiProcessorCount;
+    limits.clock_khz = prop.clockRate;
+    limits.hbm_bytes = (int64_t)prop.totalGlobalMem;
+    std::snprintf(limits.arch, sizeof(limits.arch), "%s", prop.gcnArchName);
+    g_limits_by_device[device] = limits;
+    out = limits;
     return GERN_HIP_OK;
 }
 
@@ -87,11 +91,12 @@ int compile_program(const char *source, const char *const *name_exprs, int n_nam
     }
     std::string arch_name = arch ? arch : "";
     if (arch_name.empty()) {
-        int rc = load_limits();
+        gern_hip_limits limits;
+        int rc = current_limits(limits);
         if (rc != GERN_HIP_OK) {
             return rc;
         }
-        arch_name = g_limits.arch;
+        arch_name = limits.arch;
     }
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, source, "gern_generated.hip", 0, nullptr, nullptr);
@@ -195,7 +200,8 @@ int gern_hip_compile(const char *source, const char *const *name_exprs, int n_na
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_compile: null output handle");
     }
     *out = nullptr;
-    int rc = load_limits();
+    gern_hip_limits limits;
+    int rc = current_limits(limits);
     if (rc != GERN_HIP_OK) {
         return rc;
     }
@@ -282,7 +288,8 @@ int gern_hip_launch(gern_hip_kernel kernel, const uint32_t grid[3], const uint32
     if (kernel == nullptr || grid == nullptr || block == nullptr) {
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: null argument");
     }
-    int rc = load_limits();
+    gern_hip_limits limits;
+    int rc = current_limits(limits);
     if (rc != GERN_HIP_OK) {
         return rc;
     }
@@ -291,25 +298,25 @@ int gern_hip_launch(gern_hip_kernel kernel, const uint32_t grid[3], const uint32
         if (grid[i] == 0 || block[i] == 0) {
             return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: zero-sized grid or block dimension");
         }
-        if (block[i] > (uint32_t)g_limits.max_block_dim[i]) {
+        if (block[i] > (uint32_t)limits.max_block_dim[i]) {
             return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: block dimension " + std::to_string(i) +
                                                    " = " + std::to_string(block[i]) + " exceeds the device limit");
         }
-        if (grid[i] > (uint32_t)g_limits.max_grid_dim[i]) {
+        if (grid[i] > (uint32_t)limits.max_grid_dim[i]) {
             return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: grid dimension " + std::to_string(i) +
                                                    " = " + std::to_string(grid[i]) + " exceeds the device limit");
         }
         threads *= block[i];
     }
-    if (threads > (uint64_t)g_limits.max_threads_per_block) {
+    if (threads > (uint64_t)limits.max_threads_per_block) {
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: " + std::to_string(threads) +
                                                " threads per block exceeds the device limit of " +
-                                               std::to_string(g_limits.max_threads_per_block));
+                                               std::to_string(limits.max_threads_per_block));
     }
-    if ((int64_t)lds_bytes > g_limits.lds_bytes_per_block) {
+    if ((int64_t)lds_bytes > limits.lds_bytes_per_block) {
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_launch: " + std::to_string(lds_bytes) +
                                                " bytes of LDS exceeds the per-block limit of " +
-                                               std::to_string(g_limits.lds_bytes_per_block));
+                                               std::to_string(limits.lds_bytes_per_block));
     }
     HIP_TRY(hipModuleLaunchKernel(kernel->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                   lds_bytes, (hipStream_t)stream, params, nullptr));
@@ -421,12 +428,7 @@ int gern_hip_device_limits(gern_hip_limits *out) {
     if (out == nullptr) {
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_device_limits: null output");
     }
-    int rc = load_limits();
-    if (rc != GERN_HIP_OK) {
-        return rc;
-    }
-    *out = g_limits;
-    return GERN_HIP_OK;
+    return current_limits(*out);
 }
 
 int gern_hip_device_count(int *count) {
