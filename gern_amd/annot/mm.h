@@ -15,8 +15,9 @@ namespace annot {
 class MatrixOperand : public AbstractDataType {
 public:
     enum Element { F32, BF16 };
-    // exact: the caller guarantees that the matrix extents are multiples of
-    // the window sizes the program tiles with, so windows need no bounds tests.
+    // exact: the caller guarantees what gernels::GlobalView calls EXACT (the
+    // reduction extent is a multiple of 64, rows are 16-byte aligned multiples
+    // of 8 elements); the bf16 gernel then takes its direct-to-LDS path.
     MatrixOperand(const std::string &name, Element element, bool exact = false)
         : name(name), element(element), exact(exact) {
     }

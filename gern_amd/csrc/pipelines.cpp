@@ -50,7 +50,7 @@ AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
 struct gern_pipeline_s {
     enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
-    std::unique_ptr<Runner> exact;   // GEMM bf16: the kernel for shapes that are multiples of the tile
+    std::unique_ptr<Runner> exact;   // GEMM bf16: the kernel for K % 64 == 0, N % 8 == 0
     std::string source;
     std::string kernel_name;
     std::string exact_source, exact_kernel_name;
@@ -319,8 +319,8 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                                     256, 256, lds),
                         flags);
             if (rc == 0) {
-                // The same program on data structures that promise whole tiles:
-                // eight wavefronts, no bounds tests.  That gernel keeps its two
+                // The same program on data structures that promise whole K stages:
+                // eight wavefronts, loads straight into LDS.  That gernel keeps its two
                 // stages in static LDS (gernels/mm.h, mfma_direct): no dynamic LDS.
                 gern_pipeline_s fast;
                 rc = finish(&fast,
@@ -372,9 +372,9 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    // whole tiles, and row pitches (K for A, N for B) within the fast gernel's 32-bit byte offsets
-    p->last_run_exact =
-        p->exact && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K <= (int64_t(1) << 21) && N <= (int64_t(1) << 21);
+    // whole K stages, rows of B in whole 16-byte pieces, and row pitches (K for A, N for B) within the
+    // fast gernel's 32-bit byte offsets; M and N need not be multiples of the tile
+    p->last_run_exact = p->exact && K % 64 == 0 && N % 8 == 0 && K <= (int64_t(1) << 21) && N <= (int64_t(1) << 21);
     if (p->last_run_exact) {
         runner = p->exact.get();
     }

@@ -36,8 +36,12 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 
 // A window onto a row-major matrix in HBM: at most R x C, of which
-// rows x cols lie inside the matrix.  EXACT promises that the window lies
-// wholly inside (rows == R, cols == C): gernels then skip every bounds test.
+// rows x cols lie inside the matrix.  EXACT is a promise about the matrix the
+// window was cut from, made by the program that declares the operand: its
+// reduction extent (columns of A, rows of B) is a multiple of the 64-deep
+// stage of the bf16 gernel, its rows start on 16-byte boundaries and hold a
+// multiple of 8 elements.  Windows on the bottom and right edges may still be
+// partial: rows and cols say how much of them exists.
 template<int64_t R, int64_t C, typename T, bool EXACT>
 struct GlobalView {
     const T *data;
@@ -66,13 +70,12 @@ struct MatrixBF16 {
         return GlobalView<R, C, uint16_t, false>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
                                                  c < C ? (c < 0 ? 0 : c) : C};
     }
-    // For matrices whose extents are multiples of the window: the R x C
-    // window at (x, y), or what is left of the K extent when the window is
-    // deeper than the matrix (rows / cols then still say how much).
+    // The same window for a matrix that keeps the EXACT promise of GlobalView.
     template<int64_t R, int64_t C>
     __device__ __forceinline__ GlobalView<R, C, uint16_t, true> view_exact(int64_t x, int64_t y) const {
         const int64_t r = row - x, c = col - y;
-        return GlobalView<R, C, uint16_t, true>{data + x * lda + y, lda, r < R ? r : R, c < C ? c : C};
+        return GlobalView<R, C, uint16_t, true>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
+                                                c < C ? (c < 0 ? 0 : c) : C};
     }
 };
 
@@ -193,7 +196,9 @@ constexpr int64_t mfma_lds_bytes() {
 
 namespace detail {
 
-// The fast bf16 path: 256 x 256 tile, eight wavefronts, whole tiles only.
+// The fast bf16 path: 256 x 256 tile, eight wavefronts; K a multiple of the
+// 64-deep stage, the column count of B a multiple of 8; tiles at the bottom
+// and right edges of C may be partial.
 //
 // Both operands go from global memory STRAIGHT INTO LDS (buffer_load ... lds, 16
 // bytes per lane, no register round trip, no LDS write instructions), two
@@ -217,7 +222,8 @@ namespace detail {
 //
 // Measured alternatives at 4096^3 (us): register-staged with one barrier per
 // stage 167; two wavefront groups half a stage out of phase (one computing
-// while the other moves data) 140; this one 129-133.
+// while the other moves data) 140; this one, with 64-bit lane addresses, 131;
+// as it is, 116-124.
 template<int64_t BM, int64_t BN, int64_t KC>
 __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, true> &A,
                                             const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc<BM, BN, 8> &C) {
@@ -236,7 +242,7 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     const int w = wave_in_block();
     const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
     const int nk = (int)(k_total / kMfmaBK);
-    if (nk == 0) {
+    if (nk == 0 || A.rows <= 0 || B.cols <= 0) {  // workgroup-uniform
         return;
     }
 
@@ -250,19 +256,32 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     // (64-bit lane addresses made this kernel 10 % slower).
     // Byte offsets are 32 bit: lda and ldb below kMfmaMaxLd elements.
     const int wu = __builtin_amdgcn_readfirstlane(w);
-    int lane_off_a[2], lane_off_b[2];
+    // A tile at the bottom or right edge of C has fewer than 256 valid rows of
+    // A or columns of B.  LDS slots past the edge are filled from the last
+    // valid row / 8-column chunk instead (they only feed accumulators that the
+    // insert does not write), so no load leaves the matrices.
+    const int last_row_a = (int)A.rows - 1;
+    const int last_chunk_b = ((int)B.cols - 1) / 8;
+    int lane_off_a[4], lane_off_b[2];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        // A slot: row 8 i + lane / 8 (i = 4 w + j), position lane % 8, holds
+        // chunk (lane % 8) ^ ((row >> 1) & 7) of that row
+        const int row = 8 * (wu * 4 + j) + lane / 8;
+        const int chunk_a = (lane % 8) ^ ((row >> 1) & 7);
+        const int from_row = row < last_row_a ? row : last_row_a;
+        lane_off_a[j] = (from_row * (int)A.lda + chunk_a * 8) * 2;
+    }
 #pragma unroll
     for (int odd = 0; odd < 2; odd++) {
-        // A: row 8 i + lane / 8, chunk (lane % 8) ^ ((row >> 1) & 7); B: K row
-        // 2 i + lane / 32, chunk (lane % 32) ^ (4 * (K row & 3)); i = 4 w + j
-        const int chunk_a = (lane % 8) ^ ((4 * odd + lane / 16) & 7);
-        lane_off_a[odd] = ((lane / 8) * (int)A.lda + chunk_a * 8) * 2;
+        // B slot: K row 2 i + lane / 32, position lane % 32, holds chunk
+        // (lane % 32) ^ (4 * (K row & 3)); the K row's parity class is that of j
         const int chunk_b = (lane % 32) ^ (4 * ((2 * odd + lane / 32) & 3));
-        lane_off_b[odd] = ((lane / 32) * (int)B.lda + chunk_b * 8) * 2;
+        lane_off_b[odd] = ((lane / 32) * (int)B.lda + (chunk_b < last_chunk_b ? chunk_b : last_chunk_b) * 8) * 2;
     }
     constexpr int kRawBuffer = 0x00020000;  // 32-bit raw buffer descriptor, no swizzle, no bounds beyond num_records
     const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, -1, kRawBuffer);
-    const int row_bytes_a = (int)A.lda * 2, row_bytes_b = (int)B.lda * 2;
+    const int row_bytes_b = (int)B.lda * 2;
     auto issue = [&](int kt, unsigned char *dst) {
         const int k0 = kt * (int)kMfmaBK;
         const __amdgpu_buffer_rsrc_t desc_b =
@@ -271,7 +290,7 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
-                                                     lane_off_a[j & 1], k0 * 2 + 8 * i * row_bytes_a, 0, 0);
+                                                     lane_off_a[j], k0 * 2, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -399,8 +418,6 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
     if (nk == 0) {
         return;
     }
-    // EXACT windows: whole tiles, and a K extent that is a multiple of the
-    // stage depth; nothing needs a bounds test.
 
     const int a_row = tid / (kMfmaBK / 8), a_kc = tid % (kMfmaBK / 8);
     const int b_pair = tid % (int)(BN / 2), b_g = tid / (int)(BN / 2);
@@ -417,21 +434,8 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
 
     auto fetch = [&](int kt) {
         const int64_t k0 = (int64_t)kt * kMfmaBK;
-        if constexpr (EXACT) {
-#pragma unroll
-            for (int j = 0; j < A_CHUNKS; j++) {
-                ra[j] = *reinterpret_cast<const u32x4_t *>(a_ptr + k0 + j * a_step);
-            }
-            const uint16_t *bp = b_ptr + k0 * B.lda;
-#pragma unroll
-            for (int j = 0; j < B_TASKS; j++) {
-#pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    rb[j][q] = *reinterpret_cast<const uint32_t *>(bp + j * b_step + q * b_ld);
-                }
-            }
-        } else {
-            // Ragged tile: the same accesses, each under a predicate.  A row
+        {
+            // Every access under a predicate (tiles may be ragged).  A row
             // of A is read in whole 16-byte pieces and a row of B in whole
             // column pairs (the caller guarantees K % 8 == 0 and N % 2 == 0).
 #pragma unroll

@@ -189,10 +189,13 @@ def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K):
     assert np.array_equal(_run_gemm(gpu, "bf16", aib, bib), ai @ bi)
 
 
-# Shapes made of whole 256 x 256 tiles take the eight-wavefront kernel that
+# Shapes with K % 64 == 0 and N % 8 == 0 take the eight-wavefront kernel that
 # loads straight into LDS: one K stage, an odd number of stages, several
-# column and row tiles, and a K that spans more than one 4096-deep Reduce step.
-@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 768, 128), (768, 512, 4096 + 4096 + 64)])
+# column and row tiles, a K that spans more than one 4096-deep Reduce step,
+# and partial tiles at the bottom and right edges (one row, one 8-column
+# chunk, all but one).
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 768, 128), (768, 512, 4096 + 4096 + 64),
+                                   (300, 264, 128), (1, 8, 64), (511, 504, 320), (257, 1000, 64)])
 @pytest.mark.parametrize("overwrite", [False, True])
 def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     import torch
