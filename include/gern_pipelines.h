@@ -63,8 +63,9 @@ int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows,
  * row-major, A is M x K, B is K x N, C is M x N fp32.
  * variant 0: fp32 inputs, vector-ALU FMAs.
  * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA; needs
- *            K % 8 == 0 and N % 2 == 0.  Shapes with M % 256 == N % 256 ==
- *            K % 64 == 0 take a kernel without bounds tests.
+ *            K % 8 == 0 and N % 2 == 0.  Shapes with K % 64 == 0 and
+ *            N % 8 == 0 (any M) take the faster kernel, which loads both
+ *            operands straight into LDS.
  * Composes Tile(i)(Tile(j)(Reduce(k)(matrix_multiply))) as
  * gernels/mm/kernel_3.cu:61-75 does. */
 int gern_gemm_create(int variant, int flags, gern_pipeline *out);
@@ -83,7 +84,7 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
 
 /* The generated device source (owned by the pipeline, valid until destroy).
  * A pipeline that holds more than one kernel (bf16 GEMM) reports the one its
- * last run used; before any run, the one for whole-tile shapes. */
+ * last run used; before any run, the faster one. */
 const char *gern_pipeline_source(gern_pipeline p);
 /* The name expression of the instantiated kernel, e.g. "function_7<252, 8, 3>". */
 const char *gern_pipeline_kernel_name(gern_pipeline p);
