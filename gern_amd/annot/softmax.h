@@ -141,5 +141,37 @@ protected:
     AbstractDataTypePtr output;
 };
 
+// A row-major fp32 matrix whose subsets are rows spread over the `waves`
+// wavefronts of a workgroup (gernels::BlockTile); the launch must give the
+// workgroup exactly that many wavefronts.  Roles as for MatrixF32.
+class BlockRowsF32 : public MatrixF32 {
+public:
+    BlockRowsF32(const std::string &name, Role role, int waves)
+        : MatrixF32(name, role), suffix(std::to_string(waves)) {
+    }
+    FunctionSignature getAllocateFunction() const override {
+        return FunctionSignature{
+            .name = "gernels::allocate_block_tile" + suffix,
+            .template_args = {row, col},
+        };
+    }
+    FunctionSignature getInsertFunction() const override {
+        return FunctionSignature{
+            .name = "store_block",
+            .args = {x, y},
+        };
+    }
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{
+            .name = (role == OUTPUT ? "template view_block" : "template load_block") + suffix,
+            .args = {x, y},
+            .template_args = {row, col},
+        };
+    }
+
+private:
+    std::string suffix;
+};
+
 }  // namespace annot
 }  // namespace gern

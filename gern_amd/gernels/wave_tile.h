@@ -68,6 +68,10 @@ struct FmaAcc;
 // Defined in gernels/qk_softmax.h: sixteen full rows of logits in registers.
 template<int64_t R, int64_t N>
 struct RowBlock;
+// Defined in gernels/softmax.h: R full rows spread over the NW wavefronts of a
+// workgroup.
+template<int64_t R, int64_t C, int NW>
+struct BlockTile;
 
 // Row-major fp32 matrix in HBM.  Plain aggregate: the host fills one in and
 // the launch passes it by value, so host and device layouts must agree
@@ -100,6 +104,30 @@ struct MatrixF32 {
     __device__ __forceinline__ RowBlock<R, N> view_row_block(int64_t x, int64_t y) const;
     template<int64_t R, int64_t N>
     __device__ __forceinline__ void store_row_block(int64_t x, int64_t y, const RowBlock<R, N> &t) const;
+
+    // Rows spread over the wavefronts of a workgroup (gernels/softmax.h).  The
+    // wavefront count is part of the name because the code generator pastes
+    // names and appends <rows, cols> only.
+    template<int NW, int64_t R, int64_t C>
+    __device__ __forceinline__ BlockTile<R, C, NW> load_block(int64_t x, int64_t y) const;
+    template<int NW, int64_t R, int64_t C>
+    __device__ __forceinline__ BlockTile<R, C, NW> view_block(int64_t x, int64_t y) const;
+    template<int64_t R, int64_t C, int NW>
+    __device__ __forceinline__ void store_block(int64_t x, int64_t y, const BlockTile<R, C, NW> &t) const;
+#define GERN_BLOCK_ACCESSORS(NW)                                                                     \
+    template<int64_t R, int64_t C>                                                                   \
+    __device__ __forceinline__ BlockTile<R, C, NW> load_block##NW(int64_t x, int64_t y) const {      \
+        return load_block<NW, R, C>(x, y);                                                           \
+    }                                                                                                \
+    template<int64_t R, int64_t C>                                                                   \
+    __device__ __forceinline__ BlockTile<R, C, NW> view_block##NW(int64_t x, int64_t y) const {      \
+        return view_block<NW, R, C>(x, y);                                                           \
+    }
+    GERN_BLOCK_ACCESSORS(2)
+    GERN_BLOCK_ACCESSORS(4)
+    GERN_BLOCK_ACCESSORS(8)
+    GERN_BLOCK_ACCESSORS(16)
+#undef GERN_BLOCK_ACCESSORS
 
     // Loads the R x C tile whose top-left element is (x, y).  Elements outside
     // the matrix read as 0; a tile may therefore hang over the right or bottom

@@ -52,9 +52,11 @@ int gern_blur_chain_run(gern_pipeline p, const float *in, int64_t rows, int64_t 
                         float *out, int64_t ld_out, void *stream);
 
 /* Row-wise numerically stable softmax over matrices with exactly `ncol`
- * columns: max, x - max, exp, sum, divide, fused; rows_per_wave rows are held
- * in registers by one wavefront.  The five calls are the reference's softmax
- * gernels, apps/common/annot/functions.h:9-173. */
+ * columns: max, x - max, exp, sum, divide, fused; a workgroup holds
+ * rows_per_wave rows in registers, in one wavefront or, for rows of 1024
+ * columns and more that divide into 256-column chunks, spread over 2, 4 or 8
+ * wavefronts.  The five calls are the reference's softmax gernels,
+ * apps/common/annot/functions.h:9-173. */
 int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pipeline *out);
 int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows, int64_t ld,
                      void *stream);

@@ -110,8 +110,14 @@ def test_softmax_golden_vectors(gpu, golden, name):
     assert np.max(np.abs(got - want) / want) < 1e-5
 
 
+# Widths of 1024 columns and more that divide into 256-column chunks spread a
+# row over 2, 4 or 8 wavefronts (1024 -> 2 x 512, 2048 -> 4 x 512, 3072 -> 4 x
+# 768, 4096 -> 8 x 512, 6144 -> 8 x 768, 8192 -> 8 x 1024); the others keep one
+# wavefront per row.  Row counts that leave a partial last workgroup included.
 @pytest.mark.parametrize("shape,kw", [((64, 4096), {}), ((33, 1000), {"rows_per_wave": 2}), ((5, 7), {}),
-                                      ((128, 256), {"rows_per_wave": 4}), ((16, 8192), {})])
+                                      ((128, 256), {"rows_per_wave": 4}), ((16, 8192), {}), ((37, 1024), {}),
+                                      ((21, 2048), {"rows_per_wave": 2}), ((19, 3072), {}), ((9, 6144), {}),
+                                      ((7, 4096), {"rows_per_wave": 4}), ((40, 1280), {})])
 def test_softmax_matches_oracle(gpu, oracle, shape, kw):
     x = oracle.normal(shape, 11, 0.0, 2.0)
     got = _run_softmax(gpu, x, **kw)
@@ -139,6 +145,20 @@ def test_softmax_all_negative_rows_and_constant_rows(gpu, oracle):
     want = oracle.softmax_rows(x)
     assert np.max(np.abs(got - want) / want) < 1e-5
     assert np.all(got[3] == np.float32(1.0 / 4096))
+
+
+@pytest.mark.parametrize("ncol", [1000, 4096])
+def test_softmax_rows_with_a_wide_range(gpu, oracle, ncol):
+    # differences of more than 87 from the row maximum: exp leaves the range of
+    # the fast path (results below 2^-126); both the one-wavefront and the
+    # multi-wavefront layout must then agree with the CPU's expf, denormals included
+    x = oracle.normal((12, ncol), 17, 0.0, 40.0)
+    got = _run_softmax(gpu, x)
+    want = oracle.softmax_rows(x)
+    big = want >= 1e-30
+    assert np.max(np.abs(got[big] - want[big]) / want[big]) < 1e-5
+    assert np.max(np.abs(got[~big] - want[~big])) < 1e-35
+    assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
 
 
 # ------------------------------------------------------------------ GEMM ----
