@@ -53,12 +53,18 @@ def test_blur_chain_wavefront_mapping_and_plain_order():
     assert "gern_block_x" not in src and "blockIdx.x" in src
 
 
-def test_softmax_generates_one_pass_kernel():
-    p = gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY)
+@pytest.mark.parametrize("ncol,load,threads", [(4096, "load_block8", 512), (2048, "load_block4", 256),
+                                               (1024, "load_block2", 128), (1000, "load_wave", 64),
+                                               (512, "load_wave", 64)])
+def test_softmax_generates_one_pass_kernel(ncol, load, threads):
+    # wide rows that divide into 256-column chunks are spread over the
+    # wavefronts of a workgroup; the others stay in one wavefront
+    p = gern_amd.Softmax(ncol, flags=gern_amd.COMPILE_ONLY)
     src = p.source
     for fn in ("max_row", "subtract_vec", "exp_matrix", "sum_row", "divide_vec"):
         assert "gernels::" + fn in src
-    assert src.count("load_wave") == 1  # the row is read once
+    assert src.count(load) == 1  # the row is read once
+    assert "__launch_bounds__(%d)" % threads in src
 
 
 def test_bad_arguments_are_errors():
