@@ -73,19 +73,26 @@ extern "C" __global__ void __launch_bounds__(256) gern_copy_f4(const float4 *in,
     long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) out[i] = in[i];
 }
+typedef float gern_f4 __attribute__((ext_vector_type(4)));
+extern "C" __global__ void __launch_bounds__(256) gern_copy_f4_streaming(const gern_f4 *in, gern_f4 *out, long long n)
+{
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) __builtin_nontemporal_store(in[i], out + i);
+}
 """
 
 
-def copy_calibration(torch, gern_amd, warmup, steps):
-    """A plain float4 copy of 256 MiB through the same C ABI: the HBM rate a
-    trivial kernel reaches on this device, and the kernel of known size that
-    the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+def copy_calibration(torch, gern_amd, warmup, steps, kernel="gern_copy_f4"):
+    """A plain float4 copy of 256 MiB through the same C ABI.  gern_copy_f4 is
+    the kernel of known size that the FETCH_SIZE / WRITE_SIZE counters are
+    scaled by; gern_copy_f4_streaming (nontemporal stores, as the gernels use)
+    shows the HBM rate a trivial kernel reaches on this device."""
     import ctypes as C
     hip = gern_amd.hip_lib()
     mod, ker = C.c_void_p(), C.c_void_p()
-    names = (C.c_char_p * 1)(b"gern_copy_f4")
+    names = (C.c_char_p * 1)(kernel.encode())
     if hip.gern_hip_compile(COPY_SRC.encode(), names, 1, None, 0, None, C.byref(mod)) != 0 or \
-       hip.gern_hip_get_kernel(mod, b"gern_copy_f4", C.byref(ker)) != 0:
+       hip.gern_hip_get_kernel(mod, kernel.encode(), C.byref(ker)) != 0:
         raise gern_amd.GernError(gern_amd._hip_error())
     nbytes = 256 << 20
     src = torch.ones(nbytes // 4, device="cuda")
@@ -102,7 +109,7 @@ def copy_calibration(torch, gern_amd, warmup, steps):
     wall, ev = time_launches(launch, warmup, steps, torch, gern_amd)
     assert bool((dst == 1).all())
     return {"GB/s": 2 * nbytes / (ev * 1e-3) / 1e9, "ms": ev, "frac_hbm": 2 * nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "kernel": "gern_copy_f4", "bytes_read": nbytes, "bytes_written": nbytes}
+            "kernel": kernel, "bytes_read": nbytes, "bytes_written": nbytes}
 
 
 def cpu_baseline_blur(img_np):
@@ -263,6 +270,10 @@ def main():
     if want("copy"):
         workloads["copy_256MiB"] = copy_calibration(torch, gern_amd, args.warmup, steps2)
         log("copy 256 MiB: %.1f us  %.0f GB/s" % (workloads["copy_256MiB"]["ms"] * 1e3, workloads["copy_256MiB"]["GB/s"]))
+        workloads["copy_256MiB_streaming_stores"] = copy_calibration(torch, gern_amd, args.warmup, steps2,
+                                                                     "gern_copy_f4_streaming")
+        log("copy 256 MiB, streaming stores: %.1f us  %.0f GB/s" % (workloads["copy_256MiB_streaming_stores"]["ms"] * 1e3,
+                                                                   workloads["copy_256MiB_streaming_stores"]["GB/s"]))
 
     if result is None:
         result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "", "n_gpus": 1,
