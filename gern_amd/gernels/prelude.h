@@ -55,24 +55,44 @@ __device__ __forceinline__ float div_by(float x, float d, float rcp_d) {
     return __builtin_amdgcn_div_fixupf(q, d, x);
 }
 
-// Divisors for which div_by() is bit-exact against IEEE division over all
-// finite fp32 dividends: 3 by exhaustive check on the host; powers of two
-// because x * 2^-k is already the correctly rounded quotient and the residual
-// step then rounds the exact quotient once more.  Any other divisor takes the
-// full IEEE division.
+// Division of a tap sum by the tap count.
+//
+// The reference's blur sums start at +0 (apps/common/impl/impl.h:190-250), so
+// a sum is never -0 unless it underflowed; "sum" below is that sum with the
+// leading +0 left out, which differs only when every tap is -0 (then it is -0
+// instead of +0).  quotient_of_sum<D>() returns what the reference's
+// (0 + taps...) / D gives, bit for bit:
+//
+//  * D == 3: 1/3 = c_hi + c_lo with c_hi rounded DOWN, so that c_lo > 0;
+//    t = fma(s, c_lo, +0) is the correction term, with -0 turned into +0 on
+//    the way; q = fma(s, c_hi, t) rounds the (nearly) exact quotient once.
+//    Infinities, NaNs and zeros come out as IEEE division gives them without
+//    a fix-up (inf * c_hi + inf * c_lo = inf).  Checked on the host against
+//    x / 3.0f for all 2^32 operands: identical except for dividends with
+//    2^-126 <= |x| < 2^-122, where t underflows and the quotient (a subnormal
+//    number below 4e-38) can be one unit in the last place off: callers rule
+//    that range out first (gernels/blur.h).  The previous form -- multiply,
+//    two FMAs and v_div_fixup, exact everywhere -- cost four instructions per
+//    output instead of two, and the blur chain is limited by vector-ALU issue
+//    as much as by memory.
+//  * D a power of two: s * 2^-k is exact; the FMA with +0 only turns -0 into +0.
+//  * other D: IEEE division of (0 + s).
 template<int64_t D>
 struct ExactReciprocal {
     static constexpr bool value = (D == 2 || D == 3 || D == 4 || D == 8);
 };
 
 template<int64_t D>
-__device__ __forceinline__ float div_const(float x) {
-    if constexpr (D == 1) {
-        return x;
-    } else if constexpr (ExactReciprocal<D>::value) {
-        return div_by(x, (float)D, 1.0f / (float)D);
+__device__ __forceinline__ float quotient_of_sum(float s) {
+    if constexpr (D == 3) {
+        const float c_hi = as_float(0x3EAAAAAA);  // largest float below 1/3
+        const float c_lo = as_float(0x32AAAAAB);  // 1/3 - c_hi, rounded to nearest
+        const float t = __builtin_fmaf(s, c_lo, 0.0f);
+        return __builtin_fmaf(s, c_hi, t);
+    } else if constexpr (D == 2 || D == 4 || D == 8) {
+        return __builtin_fmaf(s, 1.0f / (float)D, 0.0f);
     } else {
-        return x / (float)D;
+        return (0.0f + s) / (float)D;
     }
 }
 

@@ -368,7 +368,8 @@ void oracle_qk_softmax_rows(const uint16_t *Q, const uint16_t *Kmat, float *S, i
 }
 
 /* ------------------------------------------------------------------ */
-/* Division by a constant with one FMA correction step.                */
+/* Division by a constant with one FMA correction step: what the blur  */
+/* gernels fall back to for tiles that hold tiny values or zeros.      */
 /* ------------------------------------------------------------------ */
 float oracle_div_const_fma(float x, float d) {
     const float c = 1.0f / d;
@@ -395,6 +396,62 @@ uint64_t oracle_div_const_mismatches(float d, uint32_t lo_bits, uint32_t hi_bits
         memcpy(&gu, &got, 4);
         if (wu != gu) bad++;
     }
+    return bad;
+}
+
+/* ------------------------------------------------------------------ */
+/* Division of a tap sum by the tap count, as the HIP blur gernels do  */
+/* it (gernels/prelude.h, quotient_of_sum): restated with libm fmaf.   */
+/* ------------------------------------------------------------------ */
+float oracle_quotient_of_sum(float s, float d) {
+    if (d == 3.0f) {
+        uint32_t hi_bits = 0x3EAAAAAAu, lo_bits = 0x32AAAAABu; /* largest float below 1/3; 1/3 minus it */
+        float c_hi, c_lo;
+        memcpy(&c_hi, &hi_bits, 4);
+        memcpy(&c_lo, &lo_bits, 4);
+        float t = fmaf(s, c_lo, 0.0f);
+        return fmaf(s, c_hi, t);
+    }
+    if (d == 2.0f || d == 4.0f || d == 8.0f) {
+        return fmaf(s, 1.0f / d, 0.0f);
+    }
+    return (0.0f + s) / d;
+}
+
+/* Compares oracle_quotient_of_sum(x, d) with what the reference computes from
+ * the same sum, (0.0f + x) / d, over the bit patterns [lo_bits, hi_bits).
+ * NaNs are skipped.  Returns the number of patterns that differ bitwise;
+ * *max_ulp receives the largest difference in units in the last place and
+ * *min_abs / *max_abs the smallest and largest |x| among the differing ones. */
+uint64_t oracle_quotient_mismatches(float d, uint32_t lo_bits, uint32_t hi_bits, uint32_t *max_ulp,
+                                    float *min_abs, float *max_abs) {
+    uint64_t bad = 0;
+    uint32_t worst = 0;
+    float lo = INFINITY, hi = 0.0f;
+    for (uint64_t b = lo_bits; b < (uint64_t)hi_bits; b++) {
+        uint32_t u = (uint32_t)b;
+        float x;
+        memcpy(&x, &u, 4);
+        if (x != x) continue;
+        volatile float sum = 0.0f + x;
+        float want = sum / d;
+        float got = oracle_quotient_of_sum(x, d);
+        uint32_t wu, gu;
+        memcpy(&wu, &want, 4);
+        memcpy(&gu, &got, 4);
+        if (wu != gu) {
+            bad++;
+            /* same sign here (a sign flip would be a difference of ~2^31) */
+            uint32_t diff = wu > gu ? wu - gu : gu - wu;
+            if (diff > worst) worst = diff;
+            float ax = fabsf(x);
+            if (ax < lo) lo = ax;
+            if (ax > hi) hi = ax;
+        }
+    }
+    if (max_ulp) *max_ulp = worst;
+    if (min_abs) *min_abs = lo;
+    if (max_abs) *max_abs = hi;
     return bad;
 }
 

@@ -101,11 +101,24 @@ void oracle_qk_softmax_rows(const uint16_t *Q, const uint16_t *Kmat, float *S, i
 /* ---- division by a constant ------------------------------------------- */
 /* q = x * RN(1/d); r = fma(-d, q, x); q' = fma(r, RN(1/d), q), then the IEEE
  * result for zero / infinite / NaN dividends (what v_div_fixup_f32 does).  The
- * HIP blur gernels divide this way; this restates it with libm fmaf. */
+ * HIP blur gernels divide this way when a tile holds tiny values or zeros;
+ * this restates it with libm fmaf. */
 float oracle_div_const_fma(float x, float d);
 /* Number of fp32 bit patterns in [lo_bits, hi_bits) for which
  * oracle_div_const_fma(x,d) differs bitwise from x / d (NaNs skipped). */
 uint64_t oracle_div_const_mismatches(float d, uint32_t lo_bits, uint32_t hi_bits);
+
+/* ---- division of a tap sum by the tap count ---------------------------- */
+/* What the HIP blur gernels compute for (0 + taps...) / d from the tap sum s
+ * formed WITHOUT the leading zero (gernels/prelude.h, quotient_of_sum): for
+ * d == 3 two FMAs with 1/3 split in two floats, for powers of two one FMA.
+ * This restates it with libm fmaf so that it can be checked on the host. */
+float oracle_quotient_of_sum(float s, float d);
+/* Bit patterns in [lo_bits, hi_bits) for which oracle_quotient_of_sum(x, d)
+ * differs bitwise from the reference's (0.0f + x) / d (NaNs skipped), the
+ * largest difference in ulp, and the range of |x| where they occur. */
+uint64_t oracle_quotient_mismatches(float d, uint32_t lo_bits, uint32_t hi_bits, uint32_t *max_ulp,
+                                    float *min_abs, float *max_abs);
 
 /* ---- comparison helpers ------------------------------------------------ */
 /* Largest ulp distance between two fp32 arrays (both finite). */

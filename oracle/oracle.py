@@ -44,6 +44,9 @@ def _load():
         "oracle_qk_softmax_rows": (None, [_u16p, _u16p, _f32p, i64, i64, i64, C.c_float, i64, i64]),
         "oracle_div_const_fma": (C.c_float, [C.c_float, C.c_float]),
         "oracle_div_const_mismatches": (C.c_uint64, [C.c_float, u32, u32]),
+        "oracle_quotient_of_sum": (C.c_float, [C.c_float, C.c_float]),
+        "oracle_quotient_mismatches": (C.c_uint64, [C.c_float, u32, u32, C.POINTER(u32), C.POINTER(C.c_float),
+                                                    C.POINTER(C.c_float)]),
         "oracle_max_ulp": (u32, [_f32p, _f32p, sz]),
     }
     for name, (res, args) in sig.items():

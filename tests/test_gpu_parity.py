@@ -93,6 +93,37 @@ def test_blur_non_finite_inputs_follow_ieee(gpu, oracle):
     assert np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)])
 
 
+def test_blur_signed_zeros_and_negative_values(gpu, oracle):
+    # the reference's sums start at +0, so a neighbourhood of -0 gives +0; the
+    # kernel leaves the leading zero out of its sums and must still agree in
+    # every bit, signs of zeros included
+    img = (oracle.uniform((40, 300), 4) - np.float32(0.5)).astype(np.float32)
+    img[:12, :] = -0.0
+    img[12:20, :64] = 0.0
+    img[25, 10:13] = -0.0
+    for pattern in ("x", "y", "xy", "xyx"):
+        got = _run_blur(gpu, img, pattern)
+        want = oracle.blur_chain(img, pattern)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), pattern
+    assert not np.any(np.signbit(_run_blur(gpu, np.full((16, 300), -0.0, dtype=np.float32), "xyx")))
+
+
+def test_blur_tiny_values_and_zeros_stay_exact(gpu, oracle):
+    # the two-FMA division by 3 is IEEE-exact except for sums in
+    # [2^-126, 2^-122); tiles that could produce such sums (values below 2^-60,
+    # zeros) take the slower exact division, so every range matches bit for bit
+    base = oracle.uniform((24, 300), 6) + np.float32(0.25)
+    for scale in (2.0 ** -59, 2.0 ** -61, 2.0 ** -118, 2.0 ** -125, 2.0 ** -127, 2.0 ** -140):
+        img = (base * np.float32(scale)).astype(np.float32)
+        for pattern in ("xyx", "y"):
+            assert oracle.max_ulp(_run_blur(gpu, img, pattern), oracle.blur_chain(img, pattern)) == 0, (scale, pattern)
+    sparse = base.copy()
+    sparse[::3, ::5] = 0.0
+    sparse[7, 100:140] = np.float32(1e-37)
+    got, want = _run_blur(gpu, sparse, "xyx"), oracle.blur_chain(sparse, "xyx")
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 # --------------------------------------------------------------- softmax ----
 def _run_softmax(gpu, x, **kw):
     import torch

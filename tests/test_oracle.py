@@ -187,6 +187,39 @@ def test_oracle_matches_reference_lowering(oracle):
 
 # ------------------------------------------------- division by constant ----
 def _mismatches(args):
+    import ctypes as C
+    from oracle import oracle as o
+    d, lo, hi = args
+    ulp, amin, amax = C.c_uint32(), C.c_float(), C.c_float()
+    n = int(o.lib().oracle_quotient_mismatches(d, lo, hi, C.byref(ulp), C.byref(amin), C.byref(amax)))
+    return n, ulp.value, amin.value, amax.value
+
+
+def test_two_fma_division_by_three_matches_ieee_division():
+    """quotient_of_sum for three taps: fma(s, c_hi, fma(s, c_lo, +0)) with
+    1/3 = c_hi + c_lo.  Over ALL fp32 operands (both signs, subnormals,
+    infinities, zeros) it equals (0 + s) / 3 bit for bit, except for
+    2^-126 <= |s| < 2^-122, where the correction term underflows and the
+    subnormal quotient may be one ulp off: the blur kernels rely on exactly this."""
+    chunks = [(3.0, i << 27, min((i + 1) << 27, 0x7F800001)) for i in range(16)]
+    chunks += [(3.0, 0x80000000 + (i << 27), min(0x80000000 + ((i + 1) << 27), 0xFF800001)) for i in range(16)]
+    workers = min(8, os.cpu_count() or 1)
+    with ProcessPoolExecutor(workers) as ex:
+        results = list(ex.map(_mismatches, chunks))
+    bad = [r for r in results if r[0]]
+    assert bad, "expected the known sliver of the subnormal range"
+    assert max(r[1] for r in bad) == 1                       # one unit in the last place at most
+    assert min(r[2] for r in bad) >= 2.0 ** -126             # only dividends in [2^-126, 2^-122)
+    assert max(r[3] for r in bad) < 2.0 ** -122
+    # zero of either sign comes out as +0, as (0 + s) / 3 does; infinities stay infinite
+    import ctypes as C
+    from oracle import oracle as o
+    q = o.lib().oracle_quotient_of_sum
+    assert np.float32(q(np.float32(-0.0), 3.0)).tobytes() == np.float32(0.0).tobytes()
+    assert q(np.float32(np.inf), 3.0) == np.inf and q(np.float32(-np.inf), 3.0) == -np.inf
+
+
+def _fallback_mismatches(args):
     from oracle import oracle as o
     d, lo, hi = args
     return int(o.lib().oracle_div_const_mismatches(d, lo, hi))
@@ -194,17 +227,18 @@ def _mismatches(args):
 
 def test_fma_corrected_division_by_three_is_exact():
     """q = x*RN(1/3); q += fma(-3, q, x) * RN(1/3) equals x / 3 for EVERY finite
-    fp32 x (both signs, subnormals included): the blur kernels rely on it."""
+    fp32 x (both signs, subnormals included): the blur kernels fall back to it for tiles
+    that hold tiny values or zeros."""
     chunks = [(3.0, i << 27, min((i + 1) << 27, 0x7F800000)) for i in range(16)]
     chunks += [(3.0, 0x80000000 + (i << 27), min(0x80000000 + ((i + 1) << 27), 0xFF800000)) for i in range(16)]
     workers = min(8, os.cpu_count() or 1)
     with ProcessPoolExecutor(workers) as ex:
-        bad = sum(ex.map(_mismatches, chunks))
+        bad = sum(ex.map(_fallback_mismatches, chunks))
     assert bad == 0
 
 
-def test_fma_corrected_division_powers_of_two(oracle):
-    # sampled, including the subnormal range where a second rounding could bite
+def test_division_by_powers_of_two_is_exact(oracle):
+    # sampled, including the subnormal range (the product with 2^-k rounds as the quotient does)
     for d in (2.0, 4.0, 8.0):
-        assert oracle.lib().oracle_div_const_mismatches(d, 0, 1 << 24) == 0
-        assert oracle.lib().oracle_div_const_mismatches(d, 0x3F000000, 0x3F000000 + (1 << 22)) == 0
+        for lo, hi in ((0, 1 << 24), (0x3F000000, 0x3F000000 + (1 << 22)), (0x80000000, 0x80000000 + (1 << 24))):
+            assert oracle.lib().oracle_quotient_mismatches(d, lo, hi, None, None, None) == 0
