@@ -1,21 +1,23 @@
 // Block-cooperative GEMM gernels for gfx950.
 //
-// One workgroup of 256 threads (four wavefronts, 2 x 2) owns a BM x BN tile of
-// C.  The operands are windows onto A and B in HBM; the gernel walks their
-// shared K extent in BK-deep steps, staging each step through LDS (double
-// buffered, next step's global loads in flight while this step computes) and
-// accumulating into registers.  Two flavours:
+// One workgroup owns a BM x BN tile of C.  The operands are windows onto A and
+// B in HBM; the gernel walks their shared K extent in BK-deep steps, staging
+// each step through LDS (double buffered, next step's global loads in flight
+// while this step computes) and accumulating into registers.  Two flavours:
 //
 //   bf16 inputs, fp32 accumulation on the matrix cores
-//       v_mfma_f32_32x32x16_bf16; each wavefront owns (BM/2) x (BN/2) of C as
-//       (BM/64) x (BN/64) MFMA tiles of 16 accumulator registers.  B is
-//       row-major (K x N) but the matrix core wants K-contiguous fragments, so
-//       B is transposed on its way into LDS (dword loads of column pairs,
-//       v_perm to split them).  LDS rows are padded to 144 bytes so that the
+//       v_mfma_f32_32x32x16_bf16, MFMA tiles of 16 accumulator registers.
+//       Eight wavefronts (2 x 4) with operands loaded straight into LDS
+//       (detail::mfma_direct below) when the matrix shapes allow it; otherwise
+//       four wavefronts (2 x 2) that stage through registers: B is row-major
+//       (K x N) but the matrix core wants K-contiguous fragments, so B is
+//       transposed on its way into LDS (dword loads of column pairs, v_perm
+//       to split them), and LDS rows are padded to 144 bytes so that the
 //       16-byte fragment reads of eight consecutive lanes hit distinct banks.
 //   fp32 inputs, fp32 FMAs on the vector ALU
-//       the classic register-tiled scheme: 8 x 8 outputs per thread, A staged
-//       K-major so that both operands are read from LDS as float4.
+//       256 threads, the classic register-tiled scheme: 8 x 8 outputs per
+//       thread, A staged K-major so that both operands are read from LDS as
+//       float4.
 //
 // These replace the reference's GEMM gernels and their staging methods
 // (gernels/mm/impl/matrix_multiply.h:50-61, matrix-gpu.h:240-374): same role in
@@ -87,8 +89,9 @@ struct MatrixBF16 {
 // [wm*BM/2, ...) and columns [wn*BN/(NW/2), ...); inside a 32 x 32 MFMA tile
 // lane l, register i holds row 8*(i/4) + 4*(l/32) + i%4, column l%32.
 //
-// NW = 8 (two wavefronts per SIMD) is the fast shape: one wavefront cannot
-// issue MFMAs back to back, two interleave and hide each other's LDS waits.
+// NW = 8 (two wavefronts per SIMD) is the fast shape: a single wavefront
+// stalls on its own LDS reads, two fill each other's gaps (the SIMD gives the
+// matrix pipe to the older of the two whenever both are ready).
 template<int64_t BM, int64_t BN, int NW = 4>
 struct MfmaAcc {
     static_assert(NW == 4 || NW == 8, "four or eight wavefronts per workgroup");
