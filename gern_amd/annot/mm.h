@@ -16,8 +16,9 @@ class MatrixOperand : public AbstractDataType {
 public:
     enum Element { F32, BF16 };
     // exact: the caller guarantees what gernels::GlobalView calls EXACT (the
-    // reduction extent is a multiple of 64, rows are 16-byte aligned multiples
-    // of 8 elements); the bf16 gernel then takes its direct-to-LDS path.
+    // reduction extent is a multiple of the stage depth, 64 for bf16 and 32 for
+    // fp32; rows are 16-byte aligned whole numbers of 16-byte pieces); the
+    // matrix-core gernels then load both operands straight into LDS.
     MatrixOperand(const std::string &name, Element element, bool exact = false)
         : name(name), element(element), exact(exact) {
     }
@@ -67,9 +68,10 @@ private:
 //   FMA    fp32 FMAs, 256 threads
 //   MFMA4  matrix cores, four wavefronts (any shape)
 //   MFMA8  matrix cores, eight wavefronts (the fast shape)
+//   MFMA8_F32  fp32 operands on the matrix cores, eight wavefronts
 class MatrixAccumulator : public AbstractDataType {
 public:
-    enum Engine { FMA, MFMA4, MFMA8 };
+    enum Engine { FMA, MFMA4, MFMA8, MFMA8_F32 };
     MatrixAccumulator(const std::string &name, Engine engine, bool accumulate = true)
         : name(name), engine(engine), accumulate(accumulate) {
     }
@@ -96,9 +98,10 @@ public:
     }
     FunctionSignature getQueryFunction() const override {
         return FunctionSignature{
-            .name = engine == MFMA8   ? "template load_acc_mfma8" :
-                    engine == MFMA4 ? "template load_acc_mfma" :
-                                      "template load_acc_fma",
+            .name = engine == MFMA8_F32 ? "template load_acc_mfma8_f32" :
+                    engine == MFMA8     ? "template load_acc_mfma8" :
+                    engine == MFMA4     ? "template load_acc_mfma" :
+                                          "template load_acc_fma",
             .args = {x, y},
             .template_args = {row, col},
         };
@@ -140,10 +143,10 @@ public:
                                                              })))))
             // all threads of a workgroup cooperate
             .occupies({Grid::Unit::THREAD_X})
-            // the whole-tile bf16 gernel addresses a tile with 32-bit byte
-            // offsets (gernels/mm.h, kMfmaMaxLd)
-            .assumes(Constraint(ADTMember(A, "lda", false) <= Expr((int64_t)1 << 21)),
-                     Constraint(ADTMember(B, "lda", false) <= Expr((int64_t)1 << 21)));
+            // the matrix-core gernels address a tile with 32-bit byte offsets
+            // (gernels/mm.h): row pitches up to 2^20 elements
+            .assumes(Constraint(ADTMember(A, "lda", false) <= Expr((int64_t)1 << 20)),
+                     Constraint(ADTMember(B, "lda", false) <= Expr((int64_t)1 << 20)));
     }
     FunctionSignature getFunction() override {
         FunctionSignature f;

@@ -80,6 +80,19 @@ __global__ void __launch_bounds__(256) check_gemm_f32(gernels::MatrixF32 A, gern
 }
 template __global__ void check_gemm_f32<128, 128, 4096>(gernels::MatrixF32, gernels::MatrixF32, gernels::MatrixF32);
 
+template<int64_t BM, int64_t BN, int64_t KC>
+__global__ void __launch_bounds__(512) check_gemm_f32_mfma(gernels::MatrixF32 A, gernels::MatrixF32 B, gernels::MatrixF32 C) {
+    const int64_t i = blockIdx.y * BM, j = blockIdx.x * BN;
+    auto acc = C.template load_acc_mfma8_f32<BM, BN>(i, j);
+    for (int64_t k = 0; k < A.col; k += KC) {
+        auto a = A.template view_exact<BM, KC>(i, k);
+        auto b = B.template view_exact<KC, BN>(k, j);
+        gernels::matrix_multiply(a, b, acc);
+    }
+    C.add_acc(i, j, acc);
+}
+template __global__ void check_gemm_f32_mfma<256, 256, 4096>(gernels::MatrixF32, gernels::MatrixF32, gernels::MatrixF32);
+
 #include "gernels/qk_softmax.h"
 
 template<int64_t N, int64_t D>

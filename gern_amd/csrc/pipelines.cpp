@@ -50,7 +50,7 @@ AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
 struct gern_pipeline_s {
     enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
-    std::unique_ptr<Runner> exact;   // GEMM bf16: the kernel for K % 64 == 0, N % 8 == 0
+    std::unique_ptr<Runner> exact;   // GEMM: the direct-to-LDS matrix-core kernel (whole K stages, 16-byte row pieces)
     std::string source;
     std::string kernel_name;
     std::string exact_source, exact_kernel_name;
@@ -330,7 +330,7 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
     }
     *out = nullptr;
     if (variant != 0 && variant != 1) {
-        return fail("gern_gemm_create: variant must be 0 (fp32, vector ALU) or 1 (bf16 in, fp32 accumulate, MFMA)");
+        return fail("gern_gemm_create: variant must be 0 (fp32) or 1 (bf16 in, fp32 accumulate)");
     }
     auto p = std::make_unique<gern_pipeline_s>();
     p->kind = variant == 1 ? gern_pipeline_s::GEMM_BF16 : gern_pipeline_s::GEMM_F32;
@@ -366,6 +366,19 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                         gemmProgram(annot::MatrixOperand::F32, false, annot::MatrixAccumulator::FMA, accumulate, 128, 128,
                                     256, lds),
                         flags);
+            if (rc == 0) {
+                // fp32 on the matrix cores for matrices that promise whole K
+                // stages (gernels/mm.h, mfma_direct_f32): static LDS only.
+                gern_pipeline_s fast;
+                rc = finish(&fast,
+                            gemmProgram(annot::MatrixOperand::F32, true, annot::MatrixAccumulator::MFMA8_F32, accumulate,
+                                        256, 256, 512, 0),
+                            flags);
+                p->exact = std::move(fast.runner);
+                p->exact_source = fast.source;
+                p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
+                p->last_run_exact = true;
+            }
         }
         if (rc != 0) {
             return rc;
@@ -400,7 +413,10 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     Runner *runner = p->runner.get();
     // whole K stages, rows of B in whole 16-byte pieces, and row pitches (K for A, N for B) within the
     // fast gernel's 32-bit byte offsets; M and N need not be multiples of the tile
-    p->last_run_exact = p->exact && K % 64 == 0 && N % 8 == 0 && K <= (int64_t(1) << 21) && N <= (int64_t(1) << 21);
+    const int64_t stage = p->kind == gern_pipeline_s::GEMM_BF16 ? 64 : 32;       // K depth of an LDS stage
+    const int64_t piece = p->kind == gern_pipeline_s::GEMM_BF16 ? 8 : 4;         // elements in 16 bytes
+    const int64_t max_pitch = int64_t(1) << 20;                                   // gernels/mm.h, kMfmaMaxLd
+    p->last_run_exact = p->exact && K % stage == 0 && N % piece == 0 && K <= max_pitch && N <= max_pitch;
     if (p->last_run_exact) {
         runner = p->exact.get();
     }

@@ -40,9 +40,9 @@ extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 // A window onto a row-major matrix in HBM: at most R x C, of which
 // rows x cols lie inside the matrix.  EXACT is a promise about the matrix the
 // window was cut from, made by the program that declares the operand: its
-// reduction extent (columns of A, rows of B) is a multiple of the 64-deep
-// stage of the bf16 gernel, its rows start on 16-byte boundaries and hold a
-// multiple of 8 elements.  Windows on the bottom and right edges may still be
+// reduction extent (columns of A, rows of B) is a multiple of the LDS stage
+// depth of the matrix-core gernel (64 for bf16, 32 for fp32), its rows start
+// on 16-byte boundaries and hold a whole number of 16-byte pieces.  Windows on the bottom and right edges may still be
 // partial: rows and cols say how much of them exists.
 template<int64_t R, int64_t C, typename T, bool EXACT>
 struct GlobalView {
@@ -57,6 +57,14 @@ __device__ __forceinline__ GlobalView<R, C, float, false> MatrixF32::view(int64_
     const int64_t r = row - x, c = col - y;
     return GlobalView<R, C, float, false>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
                                           c < C ? (c < 0 ? 0 : c) : C};
+}
+
+// The same window for a matrix that keeps the EXACT promise of GlobalView.
+template<int64_t R, int64_t C>
+__device__ __forceinline__ GlobalView<R, C, float, true> MatrixF32::view_exact(int64_t x, int64_t y) const {
+    const int64_t r = row - x, c = col - y;
+    return GlobalView<R, C, float, true>{data + x * lda + y, lda, r < R ? (r < 0 ? 0 : r) : R,
+                                         c < C ? (c < 0 ? 0 : c) : C};
 }
 
 // Row-major bf16 matrix in HBM (bit patterns).
@@ -188,7 +196,7 @@ __device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const
 }
 
 constexpr int kMfmaBK = 64;                      // K depth of one LDS stage
-constexpr int64_t kMfmaMaxLd = 1 << 21;          // whole-tile bf16 path: row pitch of A and B, in elements
+constexpr int64_t kMfmaMaxLd = 1 << 20;          // direct-to-LDS paths: largest row pitch of A and B, in elements
 constexpr int kMfmaRowBytes = 2 * kMfmaBK + 16;  // padded LDS row: 144 bytes
 
 // LDS needed by matrix_multiply on bf16 operands.
@@ -579,6 +587,226 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
         }
         __syncthreads();
     }
+}
+
+// ---------------------------------------------------------------------------
+// fp32 x fp32 -> fp32 on the matrix cores
+// ---------------------------------------------------------------------------
+// v_mfma_f32_32x32x2_f32 multiplies in fp32 (no reduced-precision inputs) at
+// 256 flop per cycle and CU, twice what the vector ALU reaches without packed
+// instructions.  256 x 256 tile, eight wavefronts as 4 x 2: wavefront (wr, wc)
+// owns rows [64 wr, 64 wr + 64) as two MFMA row tiles and columns
+// [128 wc, 128 wc + 128) as four INTERLEAVED column tiles: tile tn, MFMA
+// column j is column 4 j + tn.  A lane then gets the B operands of its four
+// column tiles with one 16-byte LDS read of four consecutive columns, and
+// holds four consecutive columns of C per row: 16-byte stores.
+//
+// acc[tm][tn][i] of lane l: row 64 wr + 32 tm + 8 (i / 4) + 4 (l / 32) + i % 4,
+// column 128 wc + 4 (l % 32) + tn.
+template<int64_t BM, int64_t BN>
+struct MfmaAccF32 {
+    static_assert(BM == 256 && BN == 256, "the fp32 matrix-core gernel is written for 256 x 256 tiles");
+    static constexpr int WR = 4, WC = 2;
+    static constexpr int TM = 2, TN = 4;
+    static constexpr int threads = 8 * kWaveSize;
+    f32x16_t acc[TM][TN];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ MfmaAccF32<BM, BN> MatrixF32::load_acc_mfma8_f32(int64_t, int64_t) const {
+    MfmaAccF32<BM, BN> t;
+#pragma unroll
+    for (int tm = 0; tm < MfmaAccF32<BM, BN>::TM; tm++) {
+#pragma unroll
+        for (int tn = 0; tn < MfmaAccF32<BM, BN>::TN; tn++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                t.acc[tm][tn][i] = 0.f;
+            }
+        }
+    }
+    return t;
+}
+
+namespace detail {
+
+template<bool ADD, int64_t BM, int64_t BN>
+__device__ __forceinline__ void write_acc_f32(const MatrixF32 &m, int64_t x, int64_t y, const MfmaAccF32<BM, BN> &t) {
+    using Acc = MfmaAccF32<BM, BN>;
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int64_t r0 = x + (int64_t)(w / Acc::WC) * 64 + 4 * (lane / 32);
+    const int64_t c0 = y + (int64_t)(w % Acc::WC) * 128 + 4 * (lane % 32);
+#pragma unroll
+    for (int tm = 0; tm < Acc::TM; tm++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int64_t rr = r0 + tm * 32 + 8 * (i / 4) + (i % 4);
+            if (rr >= m.row) {
+                continue;
+            }
+            float *p = m.data + rr * m.lda + c0;
+            float4 v = make_float4(t.acc[tm][0][i], t.acc[tm][1][i], t.acc[tm][2][i], t.acc[tm][3][i]);
+            if (c0 + 3 < m.col && ((((uint64_t)p) & 15u) == 0)) {
+                if (ADD) {
+                    const float4 o = *reinterpret_cast<const float4 *>(p);
+                    v = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+                }
+                *reinterpret_cast<float4 *>(p) = v;
+            } else {
+                const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (c0 + q < m.col) {
+                        p[q] = ADD ? p[q] + e[q] : e[q];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Same structure as mfma_direct (the bf16 kernel above): both operands loaded
+// straight into LDS with scalar-addressed buffer loads, two static 64 KiB
+// stages, one barrier per stage; a stage is 32 deep in K.
+//
+//  * A stage: 256 rows x 128 bytes (32 floats); 16-byte chunk c of row m at
+//    position c ^ ((m >> 1) & 7).  Lane l of an MFMA holds row l % 32 and one
+//    of the two K indices of the instruction; lanes 0-31 take chunk 2 b, lanes
+//    32-63 chunk 2 b + 1 of K block b (8 deep), and use the chunk's four
+//    floats in four consecutive MFMAs: K index 8 b + 4 (l / 32) + j in MFMA j.
+//  * B stage: 32 K rows x 1024 bytes as they lie in memory.  For MFMA j a
+//    lane reads the four consecutive columns 128 wc + 4 (l % 32) .. + 3 of K
+//    row 8 b + 4 (l / 32) + j: one operand for each of its four column tiles.
+//  Six 16-byte LDS reads feed 32 MFMAs of 64 cycles each.
+template<int64_t BM, int64_t BN, int64_t KC>
+__device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, true> &A,
+                                                const GlobalView<KC, BN, float, true> &B, MfmaAccF32<BM, BN> &C) {
+    using Acc = MfmaAccF32<BM, BN>;
+    constexpr int BK = 32;
+    constexpr int A_BYTES = 256 * 128;
+    constexpr int STAGE = A_BYTES + BK * 1024;
+    typedef float f32x4_native __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) unsigned char stage_even_f32[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char stage_odd_f32[STAGE];
+
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
+    const int nk = (int)(k_total / BK);
+    if (nk == 0 || A.rows <= 0 || B.cols <= 0) {  // workgroup-uniform
+        return;
+    }
+    const int wu = __builtin_amdgcn_readfirstlane(w);
+    // Slots past the bottom / right edge of a partial tile are filled from the
+    // last valid row / 16-byte chunk (they feed only accumulators that the
+    // insert does not write), so no load leaves the matrices.
+    const int last_row_a = (int)A.rows - 1;
+    const int last_chunk_b = ((int)B.cols - 1) / 4;
+    int lane_off_a[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int row = 8 * (wu * 4 + j) + lane / 8;
+        const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+        lane_off_a[j] = ((row < last_row_a ? row : last_row_a) * (int)A.lda + chunk * 4) * 4;
+    }
+    const int lane_off_b = (lane < last_chunk_b ? lane : last_chunk_b) * 16;
+    constexpr int kRawBuffer = 0x00020000;
+    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, -1, kRawBuffer);
+    const int row_bytes_b = (int)B.lda * 4;
+    // Wavefront w issues A instructions 4w .. 4w+3 (8 rows each) and B
+    // instructions 4w .. 4w+3 (one K row each) of every stage.
+    auto issue = [&](int kt, unsigned char *dst) {
+        const int k0 = kt * BK;
+        const __amdgpu_buffer_rsrc_t desc_b =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(B.data + (int64_t)k0 * B.lda), 0, -1, kRawBuffer);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = wu * 4 + j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
+                                                     lane_off_a[j], k0 * 4, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = wu * 4 + j;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b,
+                                                     (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)),
+                                                     16, lane_off_b, i * row_bytes_b, 0, 0);
+        }
+    };
+
+    const int half = lane / 32;
+    const int a_row = (w / Acc::WC) * 64 + (lane % 32);
+    const int a_swz = ((lane % 32) >> 1) & 7;  // rows 64 wr + 32 tm + lane % 32: the other terms are multiples of 16
+    const int b_off = A_BYTES + (4 * half) * 1024 + ((w % Acc::WC) * 128 + 4 * (lane % 32)) * 4;
+    auto compute = [&](const unsigned char *stage) {
+#pragma unroll
+        for (int kb = 0; kb < BK / 8; kb++) {
+            f32x4_native a[Acc::TM], b[4];
+#pragma unroll
+            for (int tm = 0; tm < Acc::TM; tm++) {
+                const int at = (a_row + tm * 32) * 128 + (((2 * kb + half) ^ a_swz) * 16);
+                a[tm] = *reinterpret_cast<const f32x4_native *>(stage + at);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int at = b_off + (8 * kb + j) * 1024;
+                b[j] = *reinterpret_cast<const f32x4_native *>(stage + at);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+#pragma unroll
+                for (int tm = 0; tm < Acc::TM; tm++) {
+#pragma unroll
+                    for (int tn = 0; tn < Acc::TN; tn++) {
+                        C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][j], b[j][tn], C.acc[tm][tn], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+    auto arrive = [&]() {
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+    };
+
+    issue(0, stage_even_f32);
+    arrive();
+    for (int kt = 0; kt < nk; kt += 2) {
+        if (kt + 1 < nk) {
+            issue(kt + 1, stage_odd_f32);
+        }
+        compute(stage_even_f32);
+        arrive();
+        if (kt + 1 < nk) {
+            if (kt + 2 < nk) {
+                issue(kt + 2, stage_even_f32);
+            }
+            compute(stage_odd_f32);
+            arrive();
+        }
+    }
+}
+
+}  // namespace detail
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::add_acc(int64_t x, int64_t y, const MfmaAccF32<BM, BN> &t) const {
+    detail::write_acc_f32<true>(*this, x, y, t);
+}
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const MfmaAccF32<BM, BN> &t) const {
+    detail::write_acc_f32<false>(*this, x, y, t);
+}
+
+template<int64_t BM, int64_t BN, int64_t KC>
+__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float, true> &A,
+                                                const GlobalView<KC, BN, float, true> &B, MfmaAccF32<BM, BN> &C) {
+    detail::mfma_direct_f32(A, B, C);
 }
 
 // ---------------------------------------------------------------------------

@@ -65,6 +65,8 @@ template<int64_t BM, int64_t BN, int NW>
 struct MfmaAcc;
 template<int64_t BM, int64_t BN>
 struct FmaAcc;
+template<int64_t BM, int64_t BN>
+struct MfmaAccF32;
 // Defined in gernels/qk_softmax.h: sixteen full rows of logits in registers.
 template<int64_t R, int64_t N>
 struct RowBlock;
@@ -85,6 +87,14 @@ struct MatrixF32 {
     // GEMM operand / result access (gernels/mm.h).
     template<int64_t R, int64_t C>
     __device__ __forceinline__ GlobalView<R, C, float, false> view(int64_t x, int64_t y) const;
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ GlobalView<R, C, float, true> view_exact(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ MfmaAccF32<BM, BN> load_acc_mfma8_f32(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void add_acc(int64_t x, int64_t y, const MfmaAccF32<BM, BN> &t) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAccF32<BM, BN> &t) const;
     template<int64_t BM, int64_t BN>
     __device__ __forceinline__ MfmaAcc<BM, BN, 4> load_acc_mfma(int64_t x, int64_t y) const;
     template<int64_t BM, int64_t BN>

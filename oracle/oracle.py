@@ -130,13 +130,21 @@ def softmax_rows(x):
     return out
 
 
+def _row_range(rows, M):
+    """(first, past-the-last) row to compute; the C code writes exactly these rows."""
+    i0, i1 = (0, M) if rows is None else rows
+    if not 0 <= i0 <= i1 <= M:
+        raise ValueError("rows %r outside [0, %d]" % ((i0, i1), M))
+    return int(i0), int(i1)
+
+
 def gemm_f32(A, B, C_in=None, rows=None):
     A = np.ascontiguousarray(A, dtype=np.float32)
     B = np.ascontiguousarray(B, dtype=np.float32)
     M, K = A.shape
     N = B.shape[1]
     Cm = np.zeros((M, N), dtype=np.float32) if C_in is None else np.array(C_in, dtype=np.float32, order="C")
-    i0, i1 = (0, M) if rows is None else rows
+    i0, i1 = _row_range(rows, M)
     lib().oracle_gemm_f32_rows(A, B, Cm, M, N, K, i0, i1)
     return Cm
 
@@ -147,7 +155,7 @@ def gemm_bf16(A_bits, B_bits, rows=None):
     M, K = A_bits.shape
     N = B_bits.shape[1]
     Cm = np.zeros((M, N), dtype=np.float32)
-    i0, i1 = (0, M) if rows is None else rows
+    i0, i1 = _row_range(rows, M)
     lib().oracle_gemm_bf16_f32acc_rows(A_bits, B_bits, Cm, M, N, K, i0, i1)
     return Cm
 
@@ -158,7 +166,7 @@ def qk_softmax(Q_bits, K_bits, scale, rows=None):
     M, D = Q_bits.shape
     N = K_bits.shape[0]
     S = np.zeros((M, N), dtype=np.float32)
-    i0, i1 = (0, M) if rows is None else rows
+    i0, i1 = _row_range(rows, M)
     lib().oracle_qk_softmax_rows(Q_bits, K_bits, S, M, N, D, scale, i0, i1)
     return S
 

@@ -270,7 +270,7 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     dC = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     g(_dev(ab.view(np.int16)), _dev(bb.view(np.int16)), dC)
     torch.cuda.synchronize()
-    rows = (M - 2, M)
+    rows = (max(M - 2, 0), M)
     want = oracle.gemm_bf16(ab, bb, rows=rows)[rows[0]:rows[1]]
     got = dC.cpu().numpy()[rows[0]:rows[1]]
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
