@@ -128,6 +128,7 @@ def _kernel_notes(tmp_path, make_pipeline):
     ("blur_xyx", lambda: gern_amd.BlurChain("xyx", tile_rows=4, flags=gern_amd.COMPILE_ONLY)),
     ("softmax_4096", lambda: gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY)),
     ("gemm_f32", lambda: gern_amd.Gemm("f32", overwrite=True, flags=gern_amd.COMPILE_ONLY)),
+    ("gemm_f32_accumulate", lambda: gern_amd.Gemm("f32", flags=gern_amd.COMPILE_ONLY)),
     ("gemm_bf16", lambda: gern_amd.Gemm("bf16", overwrite=True, flags=gern_amd.COMPILE_ONLY)),
     ("gemm_bf16_accumulate", lambda: gern_amd.Gemm("bf16", flags=gern_amd.COMPILE_ONLY)),
     ("qk_softmax_4096", lambda: gern_amd.QKSoftmax(128, 4096, flags=gern_amd.COMPILE_ONLY)),
@@ -140,8 +141,9 @@ def test_headline_kernels_use_no_scratch_memory(tmp_path, name, make):
         assert k[".private_segment_fixed_size"] == 0, (name, k)
 
 
-def test_bf16_gemm_reads_one_stage_while_the_other_fills(tmp_path):
-    # The whole-tile bf16 GEMM loads stage k+1 straight into LDS while it reads
+@pytest.mark.parametrize("variant", ["bf16", "f32"])
+def test_whole_tile_gemm_reads_one_stage_while_the_other_fills(tmp_path, variant):
+    # The whole-tile GEMMs load stage k+1 straight into LDS while they read
     # stage k.  The compiler keeps the two apart only while every LDS address is
     # a short pointer chain from its own static array; when it loses track it
     # waits for all outstanding loads (a bare "s_waitcnt vmcnt(0)") before the
@@ -153,7 +155,7 @@ def test_bf16_gemm_reads_one_stage_while_the_other_fills(tmp_path):
         pytest.skip("llvm-objdump not available")
     os.environ["GERN_HIP_KEEP_DIR"] = str(tmp_path)
     try:
-        gern_amd.Gemm("bf16", overwrite=True, flags=gern_amd.COMPILE_ONLY)
+        gern_amd.Gemm(variant, overwrite=True, flags=gern_amd.COMPILE_ONLY)
     finally:
         del os.environ["GERN_HIP_KEEP_DIR"]
     checked = 0

@@ -276,6 +276,56 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
 
 
+# fp32 shapes with K % 32 == 0 and N % 4 == 0 take the eight-wavefront kernel
+# on the fp32 matrix instruction: one K stage, an odd number of stages, several
+# tiles either way, a K beyond one 4096-deep Reduce step, and partial tiles at
+# the bottom and right edges (one row, one 4-column piece, all but one).
+@pytest.mark.parametrize("M,N,K", [(256, 256, 32), (512, 256, 96), (256, 768, 64), (512, 512, 4096 + 4096 + 32),
+                                   (300, 260, 128), (1, 4, 32), (511, 508, 160), (257, 1000, 32)])
+@pytest.mark.parametrize("overwrite", [False, True])
+def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
+    import torch
+    # small integers: exact in fp32 in any order, so each element of C pins
+    # its own row of A and column of B
+    ai = np.random.RandomState(31).randint(-3, 4, size=(M, K)).astype(np.float32)
+    bi = np.random.RandomState(32).randint(-3, 4, size=(K, N)).astype(np.float32)
+    c0 = np.random.RandomState(33).randint(-5, 6, size=(M, N)).astype(np.float32)
+    g = gpu.Gemm("f32", overwrite=overwrite)
+    dC = _dev(c0)
+    g(_dev(ai), _dev(bi), dC)
+    torch.cuda.synchronize()
+    assert "256, 256" in g.kernel_name and "512" in g.kernel_name.split("<")[1].split(",")[0], g.kernel_name
+    want = ai.astype(np.float64) @ bi.astype(np.float64) + (0 if overwrite else c0)
+    assert np.array_equal(dC.cpu().numpy().astype(np.float64), want)
+    # and ordinary values against the oracle and against fp64
+    A = oracle.uniform((M, K), 41, -1.0, 1.0)
+    B = oracle.uniform((K, N), 42, -1.0, 1.0)
+    dC = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    g(_dev(A), _dev(B), dC)
+    torch.cuda.synchronize()
+    got = dC.cpu().numpy()
+    rows = (max(M - 2, 0), M)
+    want = oracle.gemm_f32(A, B, rows=rows)[rows[0]:rows[1]]
+    assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(K)
+    want64 = A.astype(np.float64) @ B.astype(np.float64)
+    assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(K)
+
+
+# Shapes the matrix-core fp32 kernel cannot take (K not a multiple of 32, N not
+# a multiple of 4) stay on the vector-ALU kernel.
+@pytest.mark.parametrize("M,N,K", [(256, 256, 48), (256, 258, 64)])
+def test_gemm_f32_other_shapes_keep_the_general_kernel(gpu, oracle, M, N, K):
+    import torch
+    ai = np.random.RandomState(51).randint(-3, 4, size=(M, K)).astype(np.float32)
+    bi = np.random.RandomState(52).randint(-3, 4, size=(K, N)).astype(np.float32)
+    g = gpu.Gemm("f32")
+    dC = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    g(_dev(ai), _dev(bi), dC)
+    torch.cuda.synchronize()
+    assert "512" not in g.kernel_name.split("<")[1].split(",")[0], g.kernel_name
+    assert np.array_equal(dC.cpu().numpy(), ai @ bi)
+
+
 @pytest.mark.parametrize("variant", ["f32", "bf16"])
 def test_gemm_accumulates_into_c(gpu, oracle, variant):
     A = oracle.uniform((192, 128), 3, -1.0, 1.0)
