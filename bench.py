@@ -245,6 +245,14 @@ def main():
         workloads["gemm_%s_4096" % variant] = {"TFLOP/s": tf, "ms": ev, "frac_peak": tf / peak, "peak_TFLOP/s": peak,
                                                "kernel": g.kernel_name}
         log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, ev * 1e3, tf, 100 * tf / peak, peak))
+        if variant == "f32":
+            # the same product on the kernel that takes every shape (vector-ALU FMAs)
+            g = gern_amd.Gemm(variant, overwrite=True, general_only=True)
+            wall, ev = time_launches(lambda: g(dA, dB, dC), 3, max(5, args.steps // 20), torch, gern_amd)
+            tf = 2.0 * n ** 3 / (ev * 1e-3) / 1e12
+            workloads["gemm_f32_4096_vector_alu"] = {"TFLOP/s": tf, "ms": ev, "frac_peak": tf / peak, "peak_TFLOP/s": peak,
+                                                     "kernel": g.kernel_name}
+            log("gemm f32 4096^3, vector-ALU kernel: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (ev * 1e3, tf, 100 * tf / peak, peak))
         del dA, dB, dC
 
     # ---- config 5: fused QK^T -> softmax ------------------------------------

@@ -18,6 +18,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 COMPILE_ONLY = 1
 NO_XCD_REMAP = 2
 GEMM_OVERWRITE = 4
+GEMM_GENERAL_ONLY = 8
 
 _libs = None
 
@@ -218,14 +219,17 @@ class Softmax(_Pipeline):
 
 
 class Gemm(_Pipeline):
-    """C += A @ B (or C = A @ B with overwrite=True).  variant "f32" (vector
-    ALU) or "bf16" (MFMA, fp32 accumulate)."""
+    """C += A @ B (or C = A @ B with overwrite=True).  variant "f32" or "bf16"
+    (fp32 accumulate); general_only=True keeps shapes that the whole-stage
+    matrix-core kernels could take on the kernel for every shape."""
 
-    def __init__(self, variant="f32", overwrite=False, flags=0):
+    def __init__(self, variant="f32", overwrite=False, general_only=False, flags=0):
         super().__init__()
         self.variant = variant
         if overwrite:
             flags |= GEMM_OVERWRITE
+        if general_only:
+            flags |= GEMM_GENERAL_ONLY
         _check(pipelines_lib().gern_gemm_create({"f32": 0, "bf16": 1}[variant], flags, C.byref(self.h)))
 
     def __call__(self, A, B, Cm, stream=None):

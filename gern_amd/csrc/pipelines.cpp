@@ -336,49 +336,35 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
     p->kind = variant == 1 ? gern_pipeline_s::GEMM_BF16 : gern_pipeline_s::GEMM_F32;
     const bool accumulate = !(flags & GERN_PIPELINE_GEMM_OVERWRITE);
     try {
-        int rc;
-        if (variant == 1) {
-            // LDS of the two pipeline stages: gernels/mm.h, mfma_lds_bytes().
-            const int64_t lds = 2 * (256 + 256) * 144;
-            rc = finish(p.get(),
-                        gemmProgram(annot::MatrixOperand::BF16, false, annot::MatrixAccumulator::MFMA4, accumulate, 256,
-                                    256, 256, lds),
+        const bool bf16 = variant == 1;
+        const auto element = bf16 ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32;
+        // The kernel for every shape.  bf16: four wavefronts, 256x256 tile, LDS of
+        // gernels/mm.h mfma_lds_bytes(); fp32: vector-ALU FMAs, 128x128 tile, LDS
+        // of fma_lds_bytes().
+        int rc = bf16 ? finish(p.get(),
+                               gemmProgram(element, false, annot::MatrixAccumulator::MFMA4, accumulate, 256, 256, 256,
+                                           2 * (256 + 256) * 144),
+                               flags)
+                      : finish(p.get(),
+                               gemmProgram(element, false, annot::MatrixAccumulator::FMA, accumulate, 128, 128, 256,
+                                           2 * 2 * 16 * 132 * 4),
+                               flags);
+        if (rc == 0 && !(flags & GERN_PIPELINE_GEMM_GENERAL_ONLY)) {
+            // The same program on data structures that promise whole K stages:
+            // eight wavefronts, 256x256 tile on the matrix cores (also for fp32),
+            // loads straight into LDS.  Those gernels keep their two stages in
+            // static LDS (gernels/mm.h, mfma_direct / mfma_direct_f32): no dynamic LDS.
+            gern_pipeline_s fast;
+            rc = finish(&fast,
+                        gemmProgram(element, true,
+                                    bf16 ? annot::MatrixAccumulator::MFMA8 : annot::MatrixAccumulator::MFMA8_F32,
+                                    accumulate, 256, 256, 512, 0),
                         flags);
-            if (rc == 0) {
-                // The same program on data structures that promise whole K stages:
-                // eight wavefronts, loads straight into LDS.  That gernel keeps its two
-                // stages in static LDS (gernels/mm.h, mfma_direct): no dynamic LDS.
-                gern_pipeline_s fast;
-                rc = finish(&fast,
-                            gemmProgram(annot::MatrixOperand::BF16, true, annot::MatrixAccumulator::MFMA8, accumulate,
-                                        256, 256, 512, 0),
-                            flags);
-                p->exact = std::move(fast.runner);
-                p->exact_source = fast.source;
-                p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
-                // The shape the pipeline is built for is the exact one.
-                p->last_run_exact = true;
-            }
-        } else {
-            // gernels/mm.h, fma_lds_bytes()
-            const int64_t lds = 2 * 2 * 16 * 132 * 4;
-            rc = finish(p.get(),
-                        gemmProgram(annot::MatrixOperand::F32, false, annot::MatrixAccumulator::FMA, accumulate, 128, 128,
-                                    256, lds),
-                        flags);
-            if (rc == 0) {
-                // fp32 on the matrix cores for matrices that promise whole K
-                // stages (gernels/mm.h, mfma_direct_f32): static LDS only.
-                gern_pipeline_s fast;
-                rc = finish(&fast,
-                            gemmProgram(annot::MatrixOperand::F32, true, annot::MatrixAccumulator::MFMA8_F32, accumulate,
-                                        256, 256, 512, 0),
-                            flags);
-                p->exact = std::move(fast.runner);
-                p->exact_source = fast.source;
-                p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
-                p->last_run_exact = true;
-            }
+            p->exact = std::move(fast.runner);
+            p->exact_source = fast.source;
+            p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
+            // The shape the pipeline is built for is the exact one.
+            p->last_run_exact = true;
         }
         if (rc != 0) {
             return rc;

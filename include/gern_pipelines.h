@@ -32,7 +32,11 @@ enum {
     /* Launch workgroups in plain blockIdx order (no XCD-aware renumbering). */
     GERN_PIPELINE_NO_XCD_REMAP = 2,
     /* GEMM only: C = A * B (C is written, never read) instead of C += A * B. */
-    GERN_PIPELINE_GEMM_OVERWRITE = 4
+    GERN_PIPELINE_GEMM_OVERWRITE = 4,
+    /* GEMM only: build and run only the kernel that takes every shape (fp32:
+     * vector-ALU FMAs; bf16: the four-wavefront kernel that stages through
+     * registers), also for shapes the whole-stage kernels could take. */
+    GERN_PIPELINE_GEMM_GENERAL_ONLY = 8
 };
 
 /* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
@@ -63,7 +67,11 @@ int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows,
 
 /* Dense GEMM C += A * B (or C = A * B with GERN_PIPELINE_GEMM_OVERWRITE),
  * row-major, A is M x K, B is K x N, C is M x N fp32.
- * variant 0: fp32 inputs, vector-ALU FMAs.
+ * variant 0: fp32 inputs and fp32 arithmetic.  Shapes with K % 32 == 0 and
+ *            N % 4 == 0 (any M) run on the fp32 matrix instruction
+ *            (v_mfma_f32_32x32x2_f32), operands loaded straight into LDS; other
+ *            shapes run on vector-ALU FMAs.  Both sum each dot product in
+ *            fp32; the order of the additions differs.
  * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA; needs
  *            K % 8 == 0 and N % 2 == 0.  Shapes with K % 64 == 0 and
  *            N % 8 == 0 (any M) take the faster kernel, which loads both
@@ -85,7 +93,7 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
                         int64_t N, float scale, void *stream);
 
 /* The generated device source (owned by the pipeline, valid until destroy).
- * A pipeline that holds more than one kernel (bf16 GEMM) reports the one its
+ * A pipeline that holds more than one kernel (the GEMMs) reports the one its
  * last run used; before any run, the faster one. */
 const char *gern_pipeline_source(gern_pipeline p);
 /* The name expression of the instantiated kernel, e.g. "function_7<252, 8, 3>". */

@@ -171,3 +171,19 @@ def test_whole_tile_gemm_reads_one_stage_while_the_other_fills(tmp_path, variant
         bare = [l for l in lines[first:last] if l.startswith("s_waitcnt") and "vmcnt(0)" in l and "lgkmcnt" not in l]
         assert not bare, bare
     assert checked == 1
+
+
+@pytest.mark.parametrize("variant", ["f32", "bf16"])
+def test_gemm_general_only_builds_one_kernel(tmp_path, variant):
+    # without the flag a GEMM pipeline holds two kernels (the whole-stage
+    # matrix-core one with 512 threads, and the one for every shape); with it,
+    # only the latter
+    os.environ["GERN_HIP_KEEP_DIR"] = str(tmp_path)
+    try:
+        g = gern_amd.Gemm(variant, general_only=True, flags=gern_amd.COMPILE_ONLY)
+    finally:
+        del os.environ["GERN_HIP_KEEP_DIR"]
+    assert len(list(tmp_path.glob("*.hsaco"))) == 1
+    assert g.kernel_name.split("<")[1].split(",")[0].strip() != "512", g.kernel_name  # <lds bytes, threads, ...>
+    both = gern_amd.Gemm(variant, flags=gern_amd.COMPILE_ONLY)
+    assert both.kernel_name.split("<")[1].split(",")[0].strip() == "512", both.kernel_name

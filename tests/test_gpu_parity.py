@@ -193,9 +193,9 @@ def test_softmax_rows_with_a_wide_range(gpu, oracle, ncol):
 
 
 # ------------------------------------------------------------------ GEMM ----
-def _run_gemm(gpu, variant, A, B, C0=None):
+def _run_gemm(gpu, variant, A, B, C0=None, general_only=False):
     import torch
-    g = gpu.Gemm(variant)
+    g = gpu.Gemm(variant, general_only=general_only)
     M, N = A.shape[0], B.shape[1]
     dC = torch.zeros((M, N), dtype=torch.float32, device="cuda") if C0 is None else _dev(C0)
     if variant == "bf16":
@@ -216,20 +216,24 @@ def test_gemm_f32_golden_and_known_answers(gpu, oracle, golden):
     assert np.array_equal(_run_gemm(gpu, "f32", a, a), golden["gemm_asc_C"])
 
 
+# general_only keeps the shapes that the matrix-core kernel could take
+# (K % 32 == 0, N % 4 == 0) on the vector-ALU kernel.
+@pytest.mark.parametrize("general_only", [False, True])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (200, 136, 72), (512, 384, 256), (1, 4, 4), (130, 260, 1032)])
-def test_gemm_f32_matches_oracle(gpu, oracle, M, N, K):
+def test_gemm_f32_matches_oracle(gpu, oracle, M, N, K, general_only):
     A = oracle.uniform((M, K), 1, -1.0, 1.0)
     B = oracle.uniform((K, N), 2, -1.0, 1.0)
-    got = _run_gemm(gpu, "f32", A, B)
+    got = _run_gemm(gpu, "f32", A, B, general_only=general_only)
     want = oracle.gemm_f32(A, B)
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(K)
 
 
+@pytest.mark.parametrize("general_only", [False, True])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (200, 136, 72), (512, 384, 256), (3, 2, 8), (130, 260, 1032)])
-def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K):
+def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K, general_only):
     ab, _ = oracle.to_bf16(oracle.uniform((M, K), 1, -1.0, 1.0))
     bb, _ = oracle.to_bf16(oracle.uniform((K, N), 2, -1.0, 1.0))
-    got = _run_gemm(gpu, "bf16", ab, bb)
+    got = _run_gemm(gpu, "bf16", ab, bb, general_only=general_only)
     want = oracle.gemm_bf16(ab, bb)
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
     # exact small integers: products and sums are exact in fp32 in any order
@@ -237,7 +241,7 @@ def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K):
     bi = np.random.RandomState(2).randint(-4, 5, size=(K, N)).astype(np.float32)
     aib, _ = oracle.to_bf16(ai)
     bib, _ = oracle.to_bf16(bi)
-    assert np.array_equal(_run_gemm(gpu, "bf16", aib, bib), ai @ bi)
+    assert np.array_equal(_run_gemm(gpu, "bf16", aib, bib, general_only=general_only), ai @ bi)
 
 
 # Shapes with K % 64 == 0 and N % 8 == 0 take the eight-wavefront kernel that
