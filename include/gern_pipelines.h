@@ -11,6 +11,11 @@
  * Plain pointers and sizes only.  Every function returns 0 on success; on
  * failure the calling thread's message is read with gern_pipelines_last_error().
  * A failure to find a GPU is an error, never a fallback.
+ *
+ * Threads: different pipelines may be created and run from different threads;
+ * one pipeline handle is for one thread at a time (a run records which of its
+ * kernels it used, and sets the stream of its Runner).  The reference's Runner
+ * is not thread-safe either (src/codegen/runner.cpp, src/codegen/codegen_printer.cpp:7: static state).
  */
 #ifndef GERN_PIPELINES_H
 #define GERN_PIPELINES_H

@@ -187,3 +187,28 @@ def test_gemm_general_only_builds_one_kernel(tmp_path, variant):
     assert g.kernel_name.split("<")[1].split(",")[0].strip() != "512", g.kernel_name  # <lds bytes, threads, ...>
     both = gern_amd.Gemm(variant, flags=gern_amd.COMPILE_ONLY)
     assert both.kernel_name.split("<")[1].split(",")[0].strip() == "512", both.kernel_name
+
+
+def test_pipelines_can_be_created_from_several_threads():
+    # creation shares only an atomic name counter and per-thread error text
+    import threading
+    results = {}
+
+    def make(i):
+        try:
+            p = gern_amd.Softmax(1024 * (i + 1), flags=gern_amd.COMPILE_ONLY) if i % 2 else \
+                gern_amd.BlurChain("xy", tile_rows=4 + i, flags=gern_amd.COMPILE_ONLY)
+            results[i] = (p.kernel_name, "__global__" in p.source)
+        except Exception as e:  # noqa: BLE001
+            results[i] = e
+
+    threads = [threading.Thread(target=make, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert len(results) == 4
+    for i, r in results.items():
+        assert not isinstance(r, Exception), (i, r)
+        assert r[1], (i, r)
+    assert len({r[0].split("<")[0] for r in results.values()}) == 4  # four distinct generated kernels
