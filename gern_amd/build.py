@@ -66,6 +66,51 @@ def build_all():
     build_cpp_tests()
 
 
+def sanitize_check():
+    """Host-side AddressSanitizer + UBSan run of the front end, the lowering and
+    the pipelines' code generation, as the reference's CI does for its CPU tests
+    (.github/workflows/main.yml:34-46).  Everything goes to build/sanitize/; the
+    in-tree libraries are left alone.  Device code is not instrumented."""
+    out = os.path.join(ROOT, "build", "sanitize")
+    os.makedirs(out, exist_ok=True)
+    san = ["-fsanitize=address,undefined", "-fno-omit-frame-pointer", "-g", "-O1"]
+    flags = [f for f in CXXFLAGS if f != "-O2"] + san
+    rpath = "-Wl,-rpath," + out + ":" + os.path.join(ROCM, "lib")
+    run(["g++"] + flags + ["-shared", os.path.join(HERE, "csrc", "gern_hip.cpp"), "-L" + os.path.join(ROCM, "lib"),
+                            "-lamdhip64", "-lhiprtc", rpath, "-o", os.path.join(out, "libgern_hip.so")])
+    srcs = sorted(glob.glob(os.path.join(HERE, "src", "*.cpp")))
+    run(["g++"] + flags + ["-shared"] + srcs + ["-L" + out, "-lgern_hip", "-ldl", rpath, "-o", os.path.join(out, "libgern.so")])
+    run(["g++"] + flags + ["-shared", os.path.join(HERE, "csrc", "pipelines.cpp"), "-L" + out, "-lgern", "-lgern_hip", "-ldl",
+                            rpath, "-o", os.path.join(out, "libgern_pipelines.so")])
+    tdir = os.path.join(ROOT, "tests", "cpp")
+    programs = []
+    for src in sorted(glob.glob(os.path.join(tdir, "test_*.cpp"))) + [os.path.join(HERE, "csrc", "sanitize_pipelines.cpp")]:
+        exe = os.path.join(out, os.path.splitext(os.path.basename(src))[0])
+        run(["g++"] + flags + ["-I" + tdir, src, "-L" + out, "-lgern_pipelines", "-lgern", "-lgern_hip", rpath, "-o", exe])
+        programs.append(exe)
+    env = dict(os.environ)
+    env.update({"GERN_TEST_LIBRARY": os.path.join(tdir, "library"), "GERN_TEST_PACKAGE": HERE,
+                "GERN_TEST_TMP": out, "GERN_TEST_COMPILE_ONLY": "1", "GERN_PACKAGE_DIR": HERE,
+                # libraries that other tools preload come before the sanitizer runtime; the JIT-compiled
+                # host functions of the CPU lowering are not instrumented; hiprtc's own allocations are not ours
+                "ASAN_OPTIONS": "verify_asan_link_order=0:detect_leaks=0:abort_on_error=0",
+                "UBSAN_OPTIONS": "print_stacktrace=1:halt_on_error=1"})
+    failed = []
+    for exe in programs:
+        print("+ " + exe, flush=True)
+        p = subprocess.run([exe], cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        bad = p.returncode != 0 or "ERROR: AddressSanitizer" in p.stdout or "runtime error:" in p.stdout
+        print(p.stdout[-3000:] if bad else "\n".join(p.stdout.splitlines()[-2:]))
+        if bad:
+            failed.append(os.path.basename(exe))
+    if failed:
+        raise SystemExit("sanitizer run failed: " + ", ".join(failed))
+    print("sanitizer run clean: " + ", ".join(os.path.basename(e) for e in programs))
+
+
 if __name__ == "__main__":
-    build_all()
+    if "--sanitize" in sys.argv[1:]:
+        sanitize_check()
+    else:
+        build_all()
     print("build ok")

@@ -31,7 +31,14 @@ int fail(const std::string &msg) {
 }
 
 // Directory that holds this library; the gernel headers live next to it.
+// Where gernels/ and annot/ are: the directory of this library, unless
+// GERN_PACKAGE_DIR names another one (a library built or installed elsewhere).
 std::string packageDir() {
+    if (const char *dir = std::getenv("GERN_PACKAGE_DIR")) {
+        if (*dir != '\0') {
+            return dir;
+        }
+    }
     Dl_info info;
     if (dladdr((const void *)&packageDir, &info) && info.dli_fname) {
         std::string path(info.dli_fname);

@@ -123,7 +123,7 @@ struct FunctionCall {
     Parameter output = Parameter();
     LaunchArguments grid;
     LaunchArguments block;
-    Access access;
+    Access access = HOST;
     Expr smem_size = Expr();
 
     FunctionCall replaceAllDS(std::map<AbstractDataTypePtr, AbstractDataTypePtr> replacement) const;
