@@ -6,12 +6,16 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <unistd.h>
+
+#include <algorithm>
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -82,6 +86,210 @@ struct CompiledProgram {
     std::map<std::string, std::string> lowered;  // name expression -> mangled name
 };
 
+// ---- optional on-disk cache of code objects (GERN_HIP_CACHE_DIR) ------------
+// The reference recompiles on every Runner::compile (src/codegen/runner.cpp:25-40,
+// seconds per pipeline).  With GERN_HIP_CACHE_DIR set, a code object is stored
+// under a 128-bit key of everything that determines it: the source text, the
+// name expressions, the options, the architecture, the hiprtc version, and the
+// content of every header the source includes with quotes (the gernels are
+// headers that the generated source includes).
+
+struct KeyHash {
+    uint64_t a = 0xcbf29ce484222325ull, b = 0x84222325cbf29ce4ull;
+    void bytes(const void *p, size_t n) {
+        const unsigned char *c = static_cast<const unsigned char *>(p);
+        for (size_t i = 0; i < n; i++) {
+            a = (a ^ c[i]) * 0x100000001b3ull;
+            b = (b ^ c[i]) * 0x9e3779b97f4a7c15ull;
+            b ^= b >> 29;
+        }
+    }
+    void text(const std::string &t) {
+        const uint64_t n = t.size();
+        bytes(&n, sizeof n);  // length-prefixed: ("ab","c") and ("a","bc") differ
+        bytes(t.data(), t.size());
+    }
+    std::string hex() const {
+        char buf[40];
+        std::snprintf(buf, sizeof buf, "%016llx%016llx", (unsigned long long)a, (unsigned long long)b);
+        return buf;
+    }
+};
+
+bool read_file(const std::string &path, std::vector<char> &out) {
+    FILE *f = std::fopen(path.c_str(), "rb");
+    if (f == nullptr) {
+        return false;
+    }
+    std::fseek(f, 0, SEEK_END);
+    const long n = std::ftell(f);
+    std::fseek(f, 0, SEEK_SET);
+    out.resize(n > 0 ? (size_t)n : 0);
+    const bool ok = n > 0 && std::fread(out.data(), 1, (size_t)n, f) == (size_t)n;
+    std::fclose(f);
+    return ok;
+}
+
+// Hashes the CONTENT of every file that `text` reaches through #include "..."
+// lines, searched first beside the including file and then in the -I
+// directories, as the compiler does.  Conditional compilation is ignored (a
+// file behind a false #if is hashed too: more misses, never a stale hit);
+// <...> headers belong to the toolchain, whose version is part of the key.
+void hash_includes(const std::string &text, const std::string &self_dir, const std::vector<std::string> &dirs,
+                   std::set<std::string> &seen, KeyHash &h, int depth) {
+    size_t pos = 0;
+    while (pos < text.size()) {
+        size_t end = text.find('\n', pos);
+        if (end == std::string::npos) {
+            end = text.size();
+        }
+        size_t i = text.find_first_not_of(" \t", pos);
+        if (i < end && text[i] == '#') {
+            i = text.find_first_not_of(" \t", i + 1);
+            if (i < end && text.compare(i, 7, "include") == 0) {
+                i = text.find_first_not_of(" \t", i + 7);
+                if (i < end && text[i] == '"') {
+                    const size_t close = text.find('"', i + 1);
+                    if (close != std::string::npos && close < end) {
+                        const std::string name = text.substr(i + 1, close - i - 1);
+                        std::vector<std::string> candidates;
+                        if (!self_dir.empty()) {
+                            candidates.push_back(self_dir + "/" + name);
+                        }
+                        for (const auto &d : dirs) {
+                            candidates.push_back(d + "/" + name);
+                        }
+                        bool found = false;
+                        for (const auto &path : candidates) {
+                            std::vector<char> content;
+                            if (!read_file(path, content)) {
+                                continue;
+                            }
+                            found = true;
+                            if (seen.insert(path).second) {
+                                const std::string body(content.begin(), content.end());
+                                h.text(name);
+                                h.text(body);
+                                if (depth < 32) {
+                                    const size_t slash = path.rfind('/');
+                                    hash_includes(body, slash == std::string::npos ? "" : path.substr(0, slash), dirs, seen, h,
+                                                  depth + 1);
+                                }
+                            }
+                            break;
+                        }
+                        if (!found) {
+                            h.text("missing " + name);
+                        }
+                    }
+                }
+            }
+        }
+        pos = end + 1;
+    }
+}
+
+std::string cache_key(const char *source, const char *const *name_exprs, int n_name_exprs,
+                      const std::vector<std::string> &options, const std::string &arch) {
+    KeyHash h;
+    h.text(source);
+    for (int i = 0; i < n_name_exprs; i++) {
+        h.text(name_exprs[i]);
+    }
+    h.text(arch);
+    int major = 0, minor = 0;
+    hiprtcVersion(&major, &minor);
+    const int version[3] = {major, minor, HIP_VERSION};
+    h.bytes(version, sizeof version);
+    std::vector<std::string> dirs;
+    for (size_t i = 0; i < options.size(); i++) {
+        h.text(options[i]);
+        std::string dir;
+        if (options[i] == "-I" && i + 1 < options.size()) {
+            dir = options[i + 1];
+        } else if (options[i].rfind("-I", 0) == 0 && options[i].size() > 2) {
+            dir = options[i].substr(2);
+            dir.erase(0, dir.find_first_not_of(' '));
+        }
+        if (!dir.empty()) {
+            dirs.push_back(dir);
+        }
+    }
+    std::set<std::string> seen;
+    hash_includes(source, "", dirs, seen, h, 0);
+    return h.hex();
+}
+
+// Entry file: "gernhip1\n", then per name expression "<expr>\n<lowered>\n",
+// then "--code <size>\n" and the code object.  Anything unexpected is a miss.
+bool cache_load(const std::string &path, const char *const *name_exprs, int n_name_exprs, CompiledProgram &out) {
+    std::vector<char> blob;
+    if (!read_file(path, blob)) {
+        return false;
+    }
+    size_t pos = 0;
+    auto line = [&](std::string &l) {
+        const void *nl = std::memchr(blob.data() + pos, '\n', blob.size() - pos);
+        if (nl == nullptr) {
+            return false;
+        }
+        const size_t end = (const char *)nl - blob.data();
+        l.assign(blob.data() + pos, end - pos);
+        pos = end + 1;
+        return true;
+    };
+    std::string l, lowered;
+    if (!line(l) || l != "gernhip1") {
+        return false;
+    }
+    std::map<std::string, std::string> names;
+    for (;;) {
+        if (!line(l)) {
+            return false;
+        }
+        if (l.rfind("--code ", 0) == 0) {
+            break;
+        }
+        if (!line(lowered)) {
+            return false;
+        }
+        names[l] = lowered;
+    }
+    const size_t size = std::strtoull(l.c_str() + 7, nullptr, 10);
+    if (size == 0 || blob.size() - pos != size || (int)names.size() > n_name_exprs) {
+        return false;
+    }
+    for (int i = 0; i < n_name_exprs; i++) {
+        if (names.find(name_exprs[i]) == names.end()) {
+            return false;
+        }
+    }
+    out.lowered = std::move(names);
+    out.code.assign(blob.begin() + pos, blob.end());
+    return true;
+}
+
+void cache_store(const std::string &path, const CompiledProgram &prog) {
+    static std::atomic<int> serial{0};
+    const std::string tmp = path + ".tmp" + std::to_string((long)getpid()) + "_" + std::to_string(serial++);
+    FILE *f = std::fopen(tmp.c_str(), "wb");
+    if (f == nullptr) {
+        return;  // a cache that cannot be written is not an error
+    }
+    bool ok = std::fputs("gernhip1\n", f) >= 0;
+    for (const auto &kv : prog.lowered) {
+        ok = ok && std::fprintf(f, "%s\n%s\n", kv.first.c_str(), kv.second.c_str()) > 0;
+    }
+    ok = ok && std::fprintf(f, "--code %zu\n", prog.code.size()) > 0;
+    ok = ok && std::fwrite(prog.code.data(), 1, prog.code.size(), f) == prog.code.size();
+    ok = (std::fclose(f) == 0) && ok;
+    if (!ok || std::rename(tmp.c_str(), path.c_str()) != 0) {  // rename: readers never see a partial entry
+        std::remove(tmp.c_str());
+    }
+}
+
+void keep_for_inspection(const char *source, const CompiledProgram &prog);
+
 int compile_program(const char *source, const char *const *name_exprs, int n_name_exprs,
                     const char *const *options, int n_options, const char *arch,
                     CompiledProgram &out) {
@@ -97,6 +305,26 @@ int compile_program(const char *source, const char *const *name_exprs, int n_nam
             return rc;
         }
         arch_name = limits.arch;
+    }
+    for (int i = 0; i < n_name_exprs; i++) {
+        if (name_exprs[i] == nullptr || std::strchr(name_exprs[i], '\n') != nullptr) {
+            return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_compile: a name expression is null or spans lines");
+        }
+    }
+    std::string cache_path;
+    if (const char *dir = std::getenv("GERN_HIP_CACHE_DIR")) {
+        if (*dir != '\0') {
+            std::vector<std::string> user_options;
+            for (int i = 0; i < n_options; i++) {
+                user_options.push_back(options[i] ? options[i] : "");
+            }
+            cache_path = std::string(dir) + "/" + cache_key(source, name_exprs, n_name_exprs, user_options, arch_name) + ".gernhip";
+            if (cache_load(cache_path, name_exprs, n_name_exprs, out)) {
+                keep_for_inspection(source, out);
+                return GERN_HIP_OK;
+            }
+            out = CompiledProgram();
+        }
     }
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, source, "gern_generated.hip", 0, nullptr, nullptr);
@@ -156,9 +384,17 @@ int compile_program(const char *source, const char *const *name_exprs, int n_nam
     out.code.resize(code_size);
     hiprtcGetCode(prog, out.code.data());
     hiprtcDestroyProgram(&prog);
-    // Like the reference Runner, which leaves its generated source and shared
-    // object in `prefix` (src/codegen/runner.cpp:20-35): with GERN_HIP_KEEP_DIR
-    // set, the source and the code object are kept there for inspection.
+    if (!cache_path.empty()) {
+        cache_store(cache_path, out);
+    }
+    keep_for_inspection(source, out);
+    return GERN_HIP_OK;
+}
+
+// Like the reference Runner, which leaves its generated source and shared
+// object in `prefix` (src/codegen/runner.cpp:20-35): with GERN_HIP_KEEP_DIR
+// set, the source and the code object are kept there for inspection.
+void keep_for_inspection(const char *source, const CompiledProgram &prog) {
     if (const char *dir = std::getenv("GERN_HIP_KEEP_DIR")) {
         static std::atomic<int> serial{0};
         const std::string base = std::string(dir) + "/gern_generated_" + std::to_string(serial++);
@@ -167,11 +403,10 @@ int compile_program(const char *source, const char *const *name_exprs, int n_nam
             std::fclose(f);
         }
         if (FILE *f = std::fopen((base + ".hsaco").c_str(), "wb")) {
-            std::fwrite(out.code.data(), 1, out.code.size(), f);
+            std::fwrite(prog.code.data(), 1, prog.code.size(), f);
             std::fclose(f);
         }
     }
-    return GERN_HIP_OK;
 }
 
 }  // namespace

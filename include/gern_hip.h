@@ -52,7 +52,13 @@ typedef struct {
  * device 0) and loads it.  `name_exprs` are C++ name expressions of the
  * __global__ templates to instantiate, e.g. "function_7<128, 8, 3>".
  * `options` are extra compiler options (e.g. "-I/path/to/gernels").
- * Replaces the `nvcc ... --shared` + dlopen step, src/codegen/runner.cpp:25-47. */
+ * Replaces the `nvcc ... --shared` + dlopen step, src/codegen/runner.cpp:25-47.
+ * With the environment variable GERN_HIP_CACHE_DIR naming an existing
+ * directory, code objects are kept there under a key of the source, the name
+ * expressions, the options, the arch, the compiler version and the content of
+ * every header the source includes with quotes; a later compile of the same
+ * inputs, in this or another process, loads the stored code object instead of
+ * compiling (the reference compiles on every Runner::compile). */
 int gern_hip_compile(const char *source, const char *const *name_exprs, int n_name_exprs,
                      const char *const *options, int n_options, const char *arch,
                      gern_hip_module *out);

@@ -212,3 +212,75 @@ def test_pipelines_can_be_created_from_several_threads():
         assert not isinstance(r, Exception), (i, r)
         assert r[1], (i, r)
     assert len({r[0].split("<")[0] for r in results.values()}) == 4  # four distinct generated kernels
+
+
+def _compile_only(src, names, options):
+    hip = gern_amd.hip_lib()
+    size = C.c_size_t()
+    arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+    opts = (C.c_char_p * len(options))(*[o.encode() for o in options])
+    rc = hip.gern_hip_compile_only(src.encode(), arr, len(names), opts, len(options), b"gfx950", C.byref(size))
+    return rc, size.value
+
+
+def test_code_object_cache(tmp_path, monkeypatch):
+    # GERN_HIP_CACHE_DIR: the second compile of the same inputs is a cache hit
+    # (no compiler run); changing the source, a name expression, an option or
+    # the content of an included header is a miss
+    import time
+    cache = tmp_path / "cache"
+    inc = tmp_path / "inc"
+    cache.mkdir()
+    inc.mkdir()
+    (inc / "scale.h").write_text("#define SCALE 2.0f\n")
+    src = '#include "scale.h"\ntemplate<int N> __global__ void k(float *p) { p[threadIdx.x] *= SCALE * N; }\n'
+    monkeypatch.setenv("GERN_HIP_CACHE_DIR", str(cache))
+    opts = ["-I" + str(inc)]
+
+    def entries():
+        return sorted(p.name for p in cache.iterdir())
+
+    t0 = time.time()
+    rc, size = _compile_only(src, ["k<3>"], opts)
+    cold = time.time() - t0
+    assert rc == 0 and size > 0 and len(entries()) == 1
+    t0 = time.time()
+    rc, size2 = _compile_only(src, ["k<3>"], opts)
+    warm = time.time() - t0
+    assert rc == 0 and size2 == size and len(entries()) == 1
+    assert warm < cold / 3, (cold, warm)
+    # each change of an input makes a new entry
+    assert _compile_only(src, ["k<4>"], opts)[0] == 0 and len(entries()) == 2
+    assert _compile_only(src + "// changed\n", ["k<3>"], opts)[0] == 0 and len(entries()) == 3
+    assert _compile_only(src, ["k<3>"], opts + ["-DUNUSED=1"])[0] == 0 and len(entries()) == 4
+    (inc / "scale.h").write_text("#define SCALE 3.0f\n")
+    assert _compile_only(src, ["k<3>"], opts)[0] == 0 and len(entries()) == 5
+    # a damaged entry is a miss and gets rewritten
+    first = cache / entries()[0]
+    for p in cache.iterdir():
+        p.write_bytes(b"gernhip1\nbroken")
+    assert _compile_only(src, ["k<3>"], opts)[0] == 0
+    assert any(p.stat().st_size > 100 for p in cache.iterdir())
+    # compile errors are not cached and still reported
+    before = entries()
+    rc, _ = _compile_only("this is not HIP", ["k<3>"], opts)
+    assert rc != 0 and entries() == before
+    del first
+
+
+def test_pipelines_use_the_code_object_cache(tmp_path, monkeypatch):
+    import time
+    monkeypatch.setenv("GERN_HIP_CACHE_DIR", str(tmp_path))
+    t0 = time.time()
+    a = gern_amd.Softmax(2048, flags=gern_amd.COMPILE_ONLY)
+    cold = time.time() - t0
+    n = len(list(tmp_path.iterdir()))
+    assert n == 1
+    t0 = time.time()
+    b = gern_amd.Softmax(2048, flags=gern_amd.COMPILE_ONLY)
+    warm = time.time() - t0
+    # generated kernels are numbered, so the second pipeline's source differs in
+    # its function name only if the generator numbers it differently
+    assert len(list(tmp_path.iterdir())) in (1, 2)
+    assert a.source and b.source
+    del cold, warm

@@ -418,3 +418,27 @@ def test_qk_softmax_full_size(gpu, oracle):
     # recover the logits' ordering from the result and compare argmax per row
     logits = (qv[:64].astype(np.float64) @ kv.T.astype(np.float64)) * float(scale)
     assert np.all(got[:64].argmax(axis=1) == logits.argmax(axis=1))
+
+
+# ------------------------------------------------- code-object cache ----
+def test_kernel_loaded_from_the_code_object_cache_runs(gpu, tmp_path, monkeypatch):
+    import ctypes as C
+    import torch
+    monkeypatch.setenv("GERN_HIP_CACHE_DIR", str(tmp_path))
+    hip = gpu.hip_lib()
+    src = b"template<int N> __global__ void scale(float *p) { p[threadIdx.x] = p[threadIdx.x] * N + 1.0f; }\n"
+    names = (C.c_char_p * 1)(b"scale<3>")
+    x = torch.arange(64, dtype=torch.float32, device="cuda")
+    expect = x.cpu().numpy()
+    for attempt in range(2):  # the first compiles and stores, the second loads the stored code object
+        mod, k = C.c_void_p(), C.c_void_p()
+        assert hip.gern_hip_compile(src, names, 1, None, 0, None, C.byref(mod)) == 0
+        assert len(list(tmp_path.iterdir())) == 1
+        assert hip.gern_hip_get_kernel(mod, b"scale<3>", C.byref(k)) == 0
+        grid, block = (C.c_uint32 * 3)(1, 1, 1), (C.c_uint32 * 3)(64, 1, 1)
+        ptr = C.c_void_p(x.data_ptr())
+        params = (C.c_void_p * 1)(C.cast(C.pointer(ptr), C.c_void_p))
+        assert hip.gern_hip_launch(k, grid, block, 0, params, None) == 0
+        torch.cuda.synchronize()
+        expect = expect * 3 + 1
+        assert np.array_equal(x.cpu().numpy(), expect), attempt
