@@ -398,18 +398,28 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     if (p->kind == gern_pipeline_s::GEMM_BF16 && ((K % 8) != 0 || (N % 2) != 0)) {
         return fail("gern_gemm_run: the bf16 path needs K % 8 == 0 and N % 2 == 0 (16-byte rows of A, dword pairs of B)");
     }
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(A), pb = reinterpret_cast<uintptr_t>(B);
+    if (p->kind == gern_pipeline_s::GEMM_BF16 ? ((pa & 15u) != 0 || (pb & 3u) != 0) : (((pa | pb) & 3u) != 0)) {
+        return fail(p->kind == gern_pipeline_s::GEMM_BF16
+                        ? "gern_gemm_run: the bf16 path reads A in 16-byte pieces and B in dwords: A must be 16-byte aligned, B 4-byte aligned"
+                        : "gern_gemm_run: A and B must be 4-byte aligned");
+    }
+    if ((reinterpret_cast<uintptr_t>(C) & 3u) != 0) {
+        return fail("gern_gemm_run: C must be 4-byte aligned");
+    }
     // MatrixF32 and MatrixBF16 share their layout.
     hip::MatrixF32 a{static_cast<float *>(const_cast<void *>(A)), M, K, K};
     hip::MatrixF32 b{static_cast<float *>(const_cast<void *>(B)), K, N, N};
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    // whole K stages, rows of B in whole 16-byte pieces, and row pitches (K for A, N for B) within the
+    // whole K stages, 16-byte aligned operands, rows of B in whole 16-byte pieces, and row pitches (K for A, N for B) within the
     // fast gernel's 32-bit byte offsets; M and N need not be multiples of the tile
     const int64_t stage = p->kind == gern_pipeline_s::GEMM_BF16 ? 64 : 32;       // K depth of an LDS stage
     const int64_t piece = p->kind == gern_pipeline_s::GEMM_BF16 ? 8 : 4;         // elements in 16 bytes
     const int64_t max_pitch = int64_t(1) << 20;                                   // gernels/mm.h, kMfmaMaxLd
-    p->last_run_exact = p->exact && K % stage == 0 && N % piece == 0 && K <= max_pitch && N <= max_pitch;
+    const bool aligned = ((pa | pb) & 15u) == 0;  // 16-byte loads
+    p->last_run_exact = p->exact && aligned && K % stage == 0 && N % piece == 0 && K <= max_pitch && N <= max_pitch;
     if (p->last_run_exact) {
         runner = p->exact.get();
     }

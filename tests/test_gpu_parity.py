@@ -367,6 +367,32 @@ def test_gemm_full_size(gpu, oracle, variant, tol):
     assert np.max(np.abs(lhs - rhs)) / np.max(np.abs(rhs)) < 1e-4
 
 
+def test_gemm_f32_operands_off_the_16_byte_grid_keep_the_general_kernel(gpu):
+    # the matrix-core kernel loads 16 bytes per lane; operands that start 4
+    # bytes off that grid are legal and take the vector-ALU kernel
+    import torch
+    M, N, K = 256, 256, 64
+    ai = np.random.RandomState(61).randint(-3, 4, size=(M, K)).astype(np.float32)
+    bi = np.random.RandomState(62).randint(-3, 4, size=(K, N)).astype(np.float32)
+    bufa = torch.zeros(M * K + 1, device="cuda")
+    bufb = torch.zeros(K * N + 1, device="cuda")
+    dA, dB = bufa[1:].view(M, K), bufb[1:].view(K, N)
+    dA.copy_(torch.from_numpy(ai))
+    dB.copy_(torch.from_numpy(bi))
+    assert dA.data_ptr() % 16 == 4 and dA.is_contiguous()
+    g = gpu.Gemm("f32")
+    dC = torch.zeros((M, N), device="cuda")
+    g(dA, dB, dC)
+    torch.cuda.synchronize()
+    assert g.kernel_name.split("<")[1].split(",")[0].strip() != "512", g.kernel_name
+    assert np.array_equal(dC.cpu().numpy(), ai @ bi)
+    # the bf16 kernels read 16-byte pieces of A: an operand off that grid is refused, not read
+    h = gpu.Gemm("bf16")
+    buf = torch.zeros(M * K + 8, dtype=torch.int16, device="cuda")
+    with pytest.raises(gpu.GernError, match="aligned"):
+        h(buf[1:1 + M * K].view(M, K), torch.zeros((K, N), dtype=torch.int16, device="cuda"), dC)
+
+
 def test_gemm_rejects_unsupported_bf16_shapes(gpu):
     import torch
     g = gpu.Gemm("bf16")
