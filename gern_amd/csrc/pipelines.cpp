@@ -494,6 +494,9 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
     if (M < 1 || N < 1 || N > p->ncol) {
         return fail("gern_qk_softmax_run: N exceeds the max_keys the pipeline was created for");
     }
+    if (((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K)) & 15u) != 0 || (reinterpret_cast<uintptr_t>(S) & 3u) != 0) {
+        return fail("gern_qk_softmax_run: Q and K are read in 16-byte pieces and must be 16-byte aligned (S 4-byte aligned)");
+    }
     hip::MatrixF32 q{reinterpret_cast<float *>(const_cast<uint16_t *>(Q)), M, p->head_dim, p->head_dim};
     hip::MatrixF32 k{reinterpret_cast<float *>(const_cast<uint16_t *>(K)), N, p->head_dim, p->head_dim};
     hip::MatrixF32 s{S, M, N, N};

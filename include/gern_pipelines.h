@@ -90,6 +90,7 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
 
 /* S = softmax_rows(scale * Q K^T): Q is M x D and K is N x D in bf16 (bit
  * patterns), S is M x N fp32; MFMA tiles feed an in-register row reduction.
+ * Q and K 16-byte aligned.
  * head_dim = D (a multiple of 32, at most 256); max_keys bounds N (a multiple
  * of 256, at most 4096: sixteen rows of logits stay in accumulators).
  * No counterpart in the reference (it has no bf16 and no matrix-core path);

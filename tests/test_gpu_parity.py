@@ -446,6 +446,18 @@ def test_qk_softmax_full_size(gpu, oracle):
     assert np.all(got[:64].argmax(axis=1) == logits.argmax(axis=1))
 
 
+def test_qk_softmax_argument_errors(gpu):
+    import torch
+    p = gpu.QKSoftmax(64, 512)
+    q = torch.zeros((16, 64), dtype=torch.int16, device="cuda")
+    k = torch.zeros((1024, 64), dtype=torch.int16, device="cuda")
+    with pytest.raises(gpu.GernError, match="max_keys"):
+        p(q, k, torch.zeros((16, 1024), device="cuda"), 1.0)
+    buf = torch.zeros(16 * 64 + 8, dtype=torch.int16, device="cuda")
+    with pytest.raises(gpu.GernError, match="aligned"):
+        p(buf[1:1 + 16 * 64].view(16, 64), k[:512], torch.zeros((16, 512), device="cuda"), 1.0)
+
+
 # ------------------------------------------------- code-object cache ----
 def test_kernel_loaded_from_the_code_object_cache_runs(gpu, tmp_path, monkeypatch):
     import ctypes as C
