@@ -5,7 +5,7 @@
 // Counterpart of the reference's apps/common/annot/adt.h:9-149.
 #pragma once
 
-#include "annotations/abstract_function.h"
+#include "annot/table.h"
 
 #include <cstdint>
 #include <string>
@@ -40,66 +40,34 @@ namespace annot {
 //   role OUTPUT : query only names the tile; the producer overwrites it and
 //                 insert stores it (clipped to the matrix)
 //   role TEMP   : never in memory; allocate makes a register tile
-class MatrixF32 : public AbstractDataType {
+class MatrixF32 : public TableADT {
 public:
     enum Role { INPUT, OUTPUT, ACCUMULATE, TEMP };
 
     MatrixF32(const std::string &name, Role role)
-        : name(name), role(role) {
+        : TableADT(name, role == TEMP ? "auto" : "gernels::MatrixF32"), role(role) {
+        fields = {x, y, row, col};
+        setCalls("gernels::allocate_wave_tile", role == OUTPUT ? "template view_wave" : "template load_wave", "store_wave");
+        query_is_written_back = role == OUTPUT || role == ACCUMULATE;
+        temporaries_are_freed = false;
     }
-    std::string getName() const override {
-        return name;
-    }
-    std::string getType() const override {
-        return role == TEMP ? "auto" : "gernels::MatrixF32";
-    }
-    std::vector<Variable> getFields() const override {
-        return {x, y, row, col};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{
-            .name = "gernels::allocate_wave_tile",
-            .template_args = {row, col},
-        };
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "destroy"};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{
-            .name = "store_wave",
-            .args = {x, y},
-        };
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{
-            .name = (role == OUTPUT) ? "template view_wave" : "template load_wave",
-            .args = {x, y},
-            .template_args = {row, col},
-        };
-    }
-    bool insertQuery() const override {
-        return role == OUTPUT || role == ACCUMULATE;
-    }
-    bool freeAlloc() const override {
-        return false;
-    }
+    // Launch dimensions are computed on the host from the caller's object.
     bool readMember(const void *object, const std::string &member, int64_t &value) const override {
         const auto *m = static_cast<const hip::MatrixF32 *>(object);
-        if (member == "row") {
-            value = m->row;
-        } else if (member == "col") {
-            value = m->col;
-        } else if (member == "lda") {
-            value = m->lda;
-        } else {
-            return false;
+        const int64_t *found = member == "row" ? &m->row : member == "col" ? &m->col : member == "lda" ? &m->lda : nullptr;
+        if (found != nullptr) {
+            value = *found;
         }
-        return true;
+        return found != nullptr;
     }
 
 protected:
-    std::string name;
+    // allocate<row, col>(), query<row, col>(x, y), insert(x, y, tile)
+    void setCalls(const std::string &allocate, const std::string &query, const std::string &insert) {
+        allocate_call = call(allocate, {}, {row, col});
+        query_call = call(query, {x, y}, {row, col});
+        insert_call = call(insert, {x, y});
+    }
     Role role;
     Variable x{"x"};
     Variable y{"y"};
@@ -108,42 +76,19 @@ protected:
 };
 
 // Per-row scalars of a tile (row maxima, row sums); always a register
-// temporary.  Fields: x origin, size.
-class WaveVec : public AbstractDataType {
+// temporary.  Fields: x origin, size.  It is never queried or inserted.
+class WaveVec : public TableADT {
 public:
     explicit WaveVec(const std::string &name)
-        : name(name) {
-    }
-    std::string getName() const override {
-        return name;
-    }
-    std::string getType() const override {
-        return "auto";
-    }
-    std::vector<Variable> getFields() const override {
-        return {x, len};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{
-            .name = "gernels::allocate_wave_vec",
-            .template_args = {len},
-        };
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "destroy"};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{.name = "unsupported_insert"};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{.name = "unsupported_query"};
-    }
-    bool freeAlloc() const override {
-        return false;
+        : TableADT(name, "auto") {
+        fields = {x, len};
+        allocate_call = call("gernels::allocate_wave_vec", {}, {len});
+        query_call = call("unsupported_query");
+        insert_call = call("unsupported_insert");
+        temporaries_are_freed = false;
     }
 
 private:
-    std::string name;
     Variable x{"x"};
     Variable len{"size", Datatype::Int64, true};
 };

@@ -6,41 +6,19 @@
 // gernels/cccl/gern_annot/functions.h:11-129.
 #pragma once
 
-#include "annotations/abstract_function.h"
+#include "annot/table.h"
 
 namespace gern {
 namespace annot {
 
-// A device pointer to one float: no fields, no query, nothing to allocate.
-class FloatPtr : public AbstractDataType {
+// A device pointer to one float: no fields, no subsets, nothing to allocate
+// (all four calls are empty).
+class FloatPtr : public TableADT {
 public:
     explicit FloatPtr(const std::string &name)
-        : name(name) {
+        : TableADT(name, "float*") {
+        free_call = FunctionSignature{};
     }
-    std::string getType() const override {
-        return "float*";
-    }
-    std::string getName() const override {
-        return name;
-    }
-    std::vector<Variable> getFields() const override {
-        return {};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{};
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{};
-    }
-
-private:
-    std::string name;
 };
 
 // Layout of the object handed to Runner::evaluate for an ArrayF32.
@@ -49,143 +27,117 @@ struct ArrayF32Layout {
     int64_t size;
 };
 
-class ArrayF32 : public AbstractDataType {
+// A float array in HBM whose subsets are per-thread register arrays of a
+// compile-time length: query copies in, insert copies back, nothing is freed.
+class ArrayF32 : public TableADT {
 public:
     ArrayF32(const std::string &name, bool temp = false)
-        : name(name), temp(temp) {
-    }
-    std::string getName() const override {
-        return name;
-    }
-    std::string getType() const override {
-        return temp ? "auto" : "gernels::ArrayF32";
-    }
-    std::vector<Variable> getFields() const override {
-        return {x, len};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{.name = "gernels::allocate_local", .template_args = {len}};
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "dummy"};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{.name = "insert_array", .args = {x}, .template_args = {len}};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{.name = "template query", .args = {x}, .template_args = {len}};
-    }
-    bool freeAlloc() const override {
-        return false;
-    }
-    bool insertQuery() const override {
-        return true;
+        : TableADT(name, temp ? "auto" : "gernels::ArrayF32") {
+        fields = {x, len};
+        allocate_call = call("gernels::allocate_local", {}, {len});
+        query_call = call("template query", {x}, {len});
+        insert_call = call("insert_array", {x}, {len});
+        free_call = call("dummy");
+        query_is_written_back = true;
+        temporaries_are_freed = false;
     }
     bool readMember(const void *object, const std::string &member, int64_t &value) const override {
-        if (member != "size") {
-            return false;
+        if (member == "size") {
+            value = static_cast<const ArrayF32Layout *>(object)->size;
         }
-        value = static_cast<const ArrayF32Layout *>(object)->size;
-        return true;
+        return member == "size";
     }
 
 private:
-    std::string name;
-    bool temp;
     Variable x{"x"};
     Variable len{"len"};
 };
 
-// *output += sum(input[0 .. k)); every workgroup reduces block_size elements
-// and adds its partial sum with one atomic.
-class GridReduce : public AbstractFunction {
+// What the three reduction gernels share: they are declared in
+// gernels/reduce.h, take (output, input) in that order, and get their sizes as
+// template arguments.
+class ReductionGernel : public AbstractFunction {
 public:
-    GridReduce()
-        : input(new const ArrayF32("input")), output(new const FloatPtr("output")) {
-    }
     FunctionSignature getFunction() override {
-        return FunctionSignature{
-            .name = "gernels::grid_reduce_total",
-            .args = {Parameter(output), Parameter(input)},
-            .template_args = {k, block_size},
-        };
-    }
-    Annotation getAnnotation() override {
-        Variable i{"i"};
-        return Computes(Produces::Subset(output, {}),
-                        Reducible(i = Expr(0), k, block_size, SubsetObj(input, {i, block_size})))
-            .occupies({Grid::Unit::THREAD_X})
-            .assumes({Grid::Dim::BLOCK_DIM_X == block_size});
+        FunctionSignature f;
+        f.name = "gernels::" + gernel;
+        f.args = {Parameter(output), Parameter(input)};
+        f.template_args = sizes();
+        return f;
     }
     std::vector<std::string> getHeader() override {
         return {"gernels/reduce.h"};
     }
 
-private:
+protected:
+    ReductionGernel(const std::string &gernel, const AbstractDataType *in, const AbstractDataType *out)
+        : input(in), output(out), gernel(gernel) {
+    }
+    virtual std::vector<Variable> sizes() const = 0;
+    // One call runs on all threads of a workgroup of exactly `block_size` threads.
+    static Annotation onWholeBlock(Pattern p, Variable block_size) {
+        return p.occupies({Grid::Unit::THREAD_X}).assumes({Grid::Dim::BLOCK_DIM_X == block_size});
+    }
+    AbstractDataTypePtr input, output;
     Variable k{"k", Datatype::Int64, true};
     Variable block_size{"block_size", Datatype::Int64, true};
-    AbstractDataTypePtr input;
-    AbstractDataTypePtr output;
+
+private:
+    std::string gernel;
+};
+
+// *output += sum(input[0 .. k)); every workgroup reduces block_size elements
+// and adds its partial sum with one atomic.
+struct GridReduce : ReductionGernel {
+    GridReduce()
+        : ReductionGernel("grid_reduce_total", new const ArrayF32("input"), new const FloatPtr("output")) {
+    }
+    Annotation getAnnotation() override {
+        Variable i{"i"};
+        return onWholeBlock(Computes(Produces::Subset(output, {}),
+                                     Reducible(i = Expr(0), k, block_size, SubsetObj(input, {i, block_size}))),
+                            block_size);
+    }
+
+protected:
+    std::vector<Variable> sizes() const override {
+        return {k, block_size};
+    }
 };
 
 // output[i] = sum of block_size consecutive inputs, one per thread.
-class BlockReduce : public AbstractFunction {
-public:
+struct BlockReduce : ReductionGernel {
     BlockReduce()
-        : input(new const ArrayF32("input")), output(new const ArrayF32("output")) {
-    }
-    FunctionSignature getFunction() override {
-        return FunctionSignature{
-            .name = "gernels::block_reduce",
-            .args = {Parameter(output), Parameter(input)},
-            .template_args = {block_size},
-        };
+        : ReductionGernel("block_reduce", new const ArrayF32("input"), new const ArrayF32("output")) {
     }
     Annotation getAnnotation() override {
-        Variable i{"i"};
-        Variable lx{"lx"};
-        return Tileable(i = Expr(0), output["size"], lx,
-                        Produces::Subset(output, {i, lx}),
-                        Consumes::Subset(input, {i * block_size * lx, block_size * lx}))
-            .occupies({Grid::Unit::THREAD_X})
-            .assumes({Grid::Dim::BLOCK_DIM_X == block_size});
-    }
-    std::vector<std::string> getHeader() override {
-        return {"gernels/reduce.h"};
+        Variable i{"i"}, lx{"lx"};
+        return onWholeBlock(Tileable(i = Expr(0), output["size"], lx, Produces::Subset(output, {i, lx}),
+                                     Consumes::Subset(input, {i * block_size * lx, block_size * lx})),
+                            block_size);
     }
 
-private:
-    Variable block_size{"block_size", Datatype::Int64, true};
-    AbstractDataTypePtr input;
-    AbstractDataTypePtr output;
+protected:
+    std::vector<Variable> sizes() const override {
+        return {block_size};
+    }
 };
 
-// *output += input[0] + ... + input[k - 1]
-class GlobalSum : public AbstractFunction {
-public:
+// *output += input[0] + ... + input[k - 1], sequentially.
+struct GlobalSum : ReductionGernel {
     GlobalSum()
-        : input(new const ArrayF32("input")), output(new const FloatPtr("output")) {
-    }
-    FunctionSignature getFunction() override {
-        return FunctionSignature{
-            .name = "gernels::global_sum",
-            .args = {Parameter(output), Parameter(input)},
-            .template_args = {k},
-        };
+        : ReductionGernel("global_sum", new const ArrayF32("input"), new const FloatPtr("output")) {
     }
     Annotation getAnnotation() override {
         Variable i{"i"};
         Variable tk{"tk", Datatype::Int64, true};
         return annotate(Computes(Produces::Subset(output, {}), Reducible(i = Expr(0), k, tk, SubsetObj(input, {i, tk}))));
     }
-    std::vector<std::string> getHeader() override {
-        return {"gernels/reduce.h"};
-    }
 
-private:
-    Variable k{"k", Datatype::Int64, true};
-    AbstractDataTypePtr input;
-    AbstractDataTypePtr output;
+protected:
+    std::vector<Variable> sizes() const override {
+        return {k};
+    }
 };
 
 }  // namespace annot

@@ -147,30 +147,12 @@ protected:
 class BlockRowsF32 : public MatrixF32 {
 public:
     BlockRowsF32(const std::string &name, Role role, int waves)
-        : MatrixF32(name, role), suffix(std::to_string(waves)) {
+        : MatrixF32(name, role) {
+        // the wavefront count is part of the gernel names: load_block8, ...
+        const std::string n = std::to_string(waves);
+        setCalls("gernels::allocate_block_tile" + n, (role == OUTPUT ? "template view_block" : "template load_block") + n,
+                 "store_block");
     }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{
-            .name = "gernels::allocate_block_tile" + suffix,
-            .template_args = {row, col},
-        };
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{
-            .name = "store_block",
-            .args = {x, y},
-        };
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{
-            .name = (role == OUTPUT ? "template view_block" : "template load_block") + suffix,
-            .args = {x, y},
-            .template_args = {row, col},
-        };
-    }
-
-private:
-    std::string suffix;
 };
 
 }  // namespace annot

@@ -75,7 +75,7 @@ int current_limits(gern_hip_limits &out) {
     limits.compute_units = prop.multiProcessorCount;
     limits.clock_khz = prop.clockRate;
     limits.hbm_bytes = (int64_t)prop.totalGlobalMem;
-    std::snprintf(limits.arch, sizeof(limits.arch), "%s", prop.gcnArchName);
+    std::snprintf(limits.arch, sizeof(limits.arch), "%.63s", prop.gcnArchName);
     g_limits_by_device[device] = limits;
     out = limits;
     return GERN_HIP_OK;

@@ -12,11 +12,14 @@ namespace gern {
 
 class AbstractFunction {
 public:
-    AbstractFunction() = default;
-    virtual ~AbstractFunction() = default;
+    // What an implementer supplies: the data-dependency annotation, the
+    // signature that calls are printed from, and the headers that declare it.
+    virtual FunctionSignature getFunction() = 0;
     virtual Annotation getAnnotation() = 0;
     virtual std::vector<std::string> getHeader() = 0;
-    virtual FunctionSignature getFunction() = 0;
+
+    AbstractFunction() = default;
+    virtual ~AbstractFunction() = default;
 
     // Binds annotation variables (by name) for the NEXT call site only.
     AbstractFunction &operator[](const std::map<std::string, Variable> &replacements) {
@@ -31,33 +34,35 @@ public:
         if (sizeof...(Args) == 0 && getFunction().args.size() != 0) {
             throw error::UserError("Called FunctionSignature " + getFunction().name + " with 0 arguments");
         }
-        return constructComposableObject(arguments);
+        return callSite(std::move(arguments));
     }
 
     template<typename FirstT, typename... Next>
     Composable construct(FirstT first, Next... remaining) {
         std::vector<Argument> arguments;
         addArguments(arguments, first, remaining...);
-        return constructComposableObject(arguments);
+        return callSite(std::move(arguments));
     }
 
 private:
-    Composable constructComposableObject(std::vector<Argument> concrete_arguments);
-    std::map<std::string, Variable> bindings;
+    // Checks the arguments against the signature, renames the annotation's
+    // variables apart, applies and clears the pending bindings.
+    Composable callSite(std::vector<Argument> concrete);
+    std::map<std::string, Variable> bindings;  // pending, for the next call site
 };
 
 class FunctionPtr : public AbstractFunction {
 public:
     FunctionPtr(Composable function, Runner::Options options,
                 std::optional<std::vector<Parameter>> ordered_parameters = std::nullopt);
-    Annotation getAnnotation() override;
-    std::vector<std::string> getHeader() override;
-    FunctionSignature getFunction() override;
+    FunctionSignature getFunction() override;      // the compiled pipeline's own signature
+    Annotation getAnnotation() override;           // the pipeline's annotation
+    std::vector<std::string> getHeader() override; // the file the pipeline was written to
 
 private:
-    Composable function;
-    Runner::Options options;
-    FunctionSignature signature;
+    Composable pipeline;
+    Runner::Options compile_options;
+    FunctionSignature compiled_signature;
 };
 
 }  // namespace gern

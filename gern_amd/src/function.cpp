@@ -166,7 +166,7 @@ std::ostream &operator<<(std::ostream &os, const MethodCall &m) {
 // ---------------------------------------------------------------------------
 // AbstractFunction
 // ---------------------------------------------------------------------------
-Composable AbstractFunction::constructComposableObject(std::vector<Argument> concrete) {
+Composable AbstractFunction::callSite(std::vector<Argument> concrete) {
     FunctionSignature f = getFunction();
     if (concrete.size() != f.args.size()) {
         throw error::UserError("Size of both arguments should be the same");
@@ -229,22 +229,22 @@ Composable AbstractFunction::constructComposableObject(std::vector<Argument> con
 
 FunctionPtr::FunctionPtr(Composable function, Runner::Options options,
                          std::optional<std::vector<Parameter>> ordered_parameters)
-    : function(function), options(options) {
+    : pipeline(function), compile_options(options) {
     Runner runner(function, ordered_parameters);
     runner.compile(options);
-    signature = runner.getSignature();
+    compiled_signature = runner.getSignature();
 }
 
 Annotation FunctionPtr::getAnnotation() {
-    return function.getAnnotation();
+    return pipeline.getAnnotation();
 }
 
 std::vector<std::string> FunctionPtr::getHeader() {
-    return {options.filename};
+    return {compile_options.filename};
 }
 
 FunctionSignature FunctionPtr::getFunction() {
-    return signature;
+    return compiled_signature;
 }
 
 }  // namespace gern

@@ -5,113 +5,72 @@
 // (test/library/array/annot/cpu-array.h:12-203).
 #pragma once
 
-#include "annotations/abstract_function.h"
-
-#include <string>
-#include <vector>
+#include "annot_table.h"
 
 namespace gern {
 namespace annot {
 
-class ArrayCPU : public AbstractDataType {
+class ArrayCPU : public TableADT {
 public:
     ArrayCPU(const std::string &name = "test")
-        : name(name) {
-    }
-    std::string getName() const override {
-        return name;
-    }
-    std::string getType() const override {
-        return "gern::impl::ArrayCPU";
-    }
-    std::vector<Variable> getFields() const override {
-        return {x, len};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{.name = "gern::impl::ArrayCPU::allocate", .args = {x, len}};
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "destroy", .args = {}};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{.name = "insert", .args = {x, len}};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{.name = "query", .args = {x, len}};
+        : TableADT(name, "gern::impl::ArrayCPU") {
+        fields = {x, len};
+        allocate_call = call("gern::impl::ArrayCPU::allocate", fields);
+        query_call = call("query", fields);
+        insert_call = call("insert", fields);
     }
     // The alternative names that Stage(...) tests swap in.
     FunctionSignature newStageFunction() const {
-        return FunctionSignature{.name = "new_stage", .args = {x, len}};
+        return call("new_stage", fields);
     }
     FunctionSignature getNewInsertFunction() const {
-        return FunctionSignature{.name = "new_insert", .args = {x, len}};
+        return call("new_insert", fields);
     }
 
 protected:
-    std::string name;
     Variable x{"x"};
     Variable len{"len"};
 };
 
-class add_1 : public AbstractFunction {
-public:
-    add_1()
-        : input(new const ArrayCPU("input")), output(new const ArrayCPU("output")) {
+struct add_1 : PiecewiseArrayFunction {
+    explicit add_1(const std::string &function = "gern::impl::add_1")
+        : PiecewiseArrayFunction(function, "array_host.h", AbstractDataTypePtr(new const ArrayCPU("input")),
+                                 AbstractDataTypePtr(new const ArrayCPU("output"))) {
     }
-    Annotation getAnnotation() override {
-        Variable x("x");
-        return annotate(Tileable(x = Expr(0), output["size"], step,
-                                 Produces::Subset(output, {x, step}),
-                                 Consumes::Subset(input, {x, step})));
-    }
-    FunctionSignature getFunction() override {
-        FunctionSignature f;
-        f.name = "gern::impl::add_1";
-        f.args = {Parameter(input), Parameter(output)};
-        return f;
-    }
-    std::vector<std::string> getHeader() override {
-        return {"array_host.h"};
-    }
-
-protected:
-    AbstractDataTypePtr input;
-    AbstractDataTypePtr output;
-    Variable step{"step"};
 };
 
-class add_1_float : public add_1 {
-public:
-    FunctionSignature getFunction() override {
-        FunctionSignature f;
-        f.name = "gern::impl::add_1_float";
-        f.args = {Parameter(input), Parameter(output), Parameter(float_val)};
-        return f;
+struct add_1_float : add_1 {
+    add_1_float()
+        : add_1("gern::impl::add_1_float") {
     }
 
 protected:
+    std::vector<Variable> trailing_arguments() const override {
+        return {float_val};
+    }
     Variable float_val{"float_val", Datatype::Float32};
 };
 
-class add1Template : public add_1 {
-public:
-    FunctionSignature getFunction() override {
-        FunctionSignature f;
-        f.name = "gern::impl::add1Template";
-        f.args = {Parameter(input), Parameter(output)};
-        f.template_args = {step};
-        return f;
+struct add1Template : add_1 {
+    add1Template()
+        : add_1("gern::impl::add1Template") {
+    }
+
+protected:
+    bool step_is_a_template_argument() const override {
+        return true;
     }
 };
 
 // Takes its step as a third argument; only call-site checks use it.
-class addWithSize : public add_1 {
-public:
-    FunctionSignature getFunction() override {
-        FunctionSignature f;
-        f.name = "gern::impl::addWithSize";
-        f.args = {Parameter(input), Parameter(output), Parameter(step)};
-        return f;
+struct addWithSize : add_1 {
+    addWithSize()
+        : add_1("gern::impl::addWithSize") {
+    }
+
+protected:
+    std::vector<Variable> trailing_arguments() const override {
+        return {step};
     }
 };
 

@@ -15,58 +15,38 @@ struct ArrayGPULayout {
     int64_t size;
 };
 
-class ArrayGPU : public AbstractDataType {
+class ArrayGPU : public TableADT {
 public:
     ArrayGPU(const std::string &name = "test")
-        : name(name) {
+        : TableADT(name, "gern::impl::ArrayGPU") {
+        fields = {x, len};
+        allocate_call = call("gern::impl::ArrayGPU::allocate", fields);
+        query_call = call("query", fields);
+        insert_call = call("insert", fields);
     }
-    std::string getName() const override {
-        return name;
-    }
-    std::string getType() const override {
-        return "gern::impl::ArrayGPU";
-    }
-    std::vector<Variable> getFields() const override {
-        return {x, len};
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{.name = "gern::impl::ArrayGPU::allocate", .args = {x, len}};
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "destroy"};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{.name = "insert", .args = {x, len}};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{.name = "query", .args = {x, len}};
-    }
+    // The launch is sized on the host from the caller's object.
     bool readMember(const void *object, const std::string &member, int64_t &value) const override {
-        if (member != "size") {
-            return false;
+        if (member == "size") {
+            value = static_cast<const ArrayGPULayout *>(object)->size;
         }
-        value = static_cast<const ArrayGPULayout *>(object)->size;
-        return true;
+        return member == "size";
     }
 
 protected:
-    std::string name;
     Variable x{"x"};
     Variable len{"len"};
 };
 
-// A scalar-unit device function.
-class Add1GPU : public add_1 {
-public:
-    Annotation getAnnotation() override {
-        Variable x("x");
-        return Tileable(x = Expr(0), output["size"], step,
-                        Produces::Subset(output, {x, step}),
-                        Consumes::Subset(input, {x, step}))
-            .occupies({Grid::Unit::SCALAR_UNIT});
+// A device function that one thread runs alone (SCALAR_UNIT).
+struct Add1GPU : PiecewiseArrayFunction {
+    Add1GPU()
+        : PiecewiseArrayFunction("gern::impl::add_1", "array_device.h", AbstractDataTypePtr(new const ArrayCPU("input")),
+                                 AbstractDataTypePtr(new const ArrayCPU("output"))) {
     }
-    std::vector<std::string> getHeader() override {
-        return {"array_device.h"};
+
+protected:
+    std::set<Grid::Unit> occupied_units() const override {
+        return {Grid::Unit::SCALAR_UNIT};
     }
 };
 
@@ -99,46 +79,25 @@ private:
 };
 
 // Subsets are register arrays of a compile-time length, copied in by query
-// and written back by insert.
+// and written back by insert; a temporary is typed `auto` and never freed.
 class ArrayStaticGPU : public ArrayGPU {
 public:
     ArrayStaticGPU(const std::string &name, bool temp = false)
-        : ArrayGPU(name), temp(temp) {
+        : ArrayGPU(name) {
+        type_name = temp ? "auto" : "gern::impl::ArrayGPU";
+        allocate_call = call("gern::impl::allocate_local", {}, {len});
+        query_call = call("query", {x}, {len});
+        insert_call = call("insert_array", {x}, {len});
+        free_call = call("dummy");
+        query_is_written_back = true;
+        temporaries_are_freed = false;
     }
-    std::string getType() const override {
-        return temp ? "auto" : "gern::impl::ArrayGPU";
-    }
-    FunctionSignature getAllocateFunction() const override {
-        return FunctionSignature{.name = "gern::impl::allocate_local", .template_args = {len}};
-    }
-    FunctionSignature getFreeFunction() const override {
-        return FunctionSignature{.name = "dummy"};
-    }
-    FunctionSignature getInsertFunction() const override {
-        return FunctionSignature{.name = "insert_array", .args = {x}, .template_args = {len}};
-    }
-    FunctionSignature getQueryFunction() const override {
-        return FunctionSignature{.name = "query", .args = {x}, .template_args = {len}};
-    }
-    bool freeAlloc() const override {
-        return false;
-    }
-    bool insertQuery() const override {
-        return true;
-    }
-
-private:
-    bool temp;
 };
 
-class Add1GPUTemplate : public Add1GPU {
-public:
-    FunctionSignature getFunction() override {
-        FunctionSignature f;
-        f.name = "gern::impl::add_1";
-        f.args = {Parameter(input), Parameter(output)};
-        f.template_args = {step};
-        return f;
+struct Add1GPUTemplate : Add1GPU {
+protected:
+    bool step_is_a_template_argument() const override {
+        return true;
     }
 };
 

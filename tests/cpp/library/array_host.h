@@ -7,9 +7,11 @@
 // allocate is a zeroed fresh array, insert copies a sub-range back.
 #pragma once
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <numeric>
 
 namespace gern {
 namespace impl {
@@ -46,42 +48,38 @@ struct ArrayCPU {
         data = nullptr;
     }
     void fill(float v) {
-        for (int64_t i = 0; i < size; i++) {
-            data[i] = v;
-        }
+        std::fill_n(data, size, v);
     }
     void ascending() {
-        for (int64_t i = 0; i < size; i++) {
-            data[i] = static_cast<float>(i);
-        }
+        std::iota(data, data + size, 0.0f);
     }
 };
 
+namespace detail {
+// out[i] = in[i] + delta for the first n elements
+inline void add_constant(const ArrayCPU &in, ArrayCPU &out, int64_t n, float delta) {
+    std::transform(in.data, in.data + n, out.data, [delta](float v) { return v + delta; });
+}
+}  // namespace detail
+
 inline void add_1(ArrayCPU in, ArrayCPU out) {
-    for (int64_t i = 0; i < in.size; i++) {
-        out.data[i] = in.data[i] + 1.0f;
-    }
+    detail::add_constant(in, out, in.size, 1.0f);
 }
 
 template<int64_t Len>
 inline void add1Template(ArrayCPU in, ArrayCPU out) {
-    for (int64_t i = 0; i < Len; i++) {
-        out.data[i] = in.data[i] + 1.0f;
-    }
+    detail::add_constant(in, out, Len, 1.0f);
 }
 
 inline void add_1_float(ArrayCPU in, ArrayCPU out, float f) {
-    for (int64_t i = 0; i < in.size; i++) {
-        out.data[i] = in.data[i] + f;
-    }
+    detail::add_constant(in, out, in.size, f);
 }
 
-// out[i] += sum of the first k entries of `in`, for every i of `out`.
+// Every element of `out` grows by in[0] + ... + in[k - 1], added one term at a
+// time (left to right, in fp32) to the element itself.
 inline void reduction(ArrayCPU in, ArrayCPU out, int64_t k) {
-    for (int64_t i = 0; i < out.size; i++) {
-        for (int64_t j = 0; j < k; j++) {
-            out.data[i] += in.data[j];
-        }
+    for (float *o = out.data; o != out.data + out.size; ++o) {
+        *o = std::accumulate(in.data, in.data + k, *o);
     }
 }
 

@@ -5,49 +5,46 @@
 // (test/library/array/impl/cpu-array-template.h).
 #pragma once
 
+#include <algorithm>
 #include <cstdint>
+#include <numeric>
 
 namespace gern {
 namespace impl {
 
 template<int64_t Size>
 struct ArrayCPUTemplate {
-    float data[Size] = {0};
     static constexpr int64_t size = Size;
+    float data[Size] = {0};
 
+    // elements [start, start + Len) as a value
     template<int64_t Len>
     ArrayCPUTemplate<Len> query(int64_t start) const {
         ArrayCPUTemplate<Len> part;
-        for (int64_t i = 0; i < Len; i++) {
-            part.data[i] = data[start + i];
-        }
+        std::copy_n(data + start, Len, part.data);
         return part;
     }
+    // ... and back
     template<int64_t Len>
     void insert(int64_t start, const ArrayCPUTemplate<Len> &part) {
-        for (int64_t i = 0; i < Len; i++) {
-            data[start + i] = part.data[i];
-        }
+        std::copy_n(part.data, Len, data + start);
     }
     void destroy() {
     }
+    // 0, 1, 2, ...
     void ascending() {
-        for (int64_t i = 0; i < Size; i++) {
-            data[i] = static_cast<float>(i);
-        }
+        std::iota(data, data + Size, 0.0f);
     }
 };
 
 template<int64_t Len>
 inline ArrayCPUTemplate<Len> temp_allocate() {
-    return ArrayCPUTemplate<Len>();
+    return {};
 }
 
 template<int64_t Len, typename In, typename Out>
 inline void add(const In &in, Out &out) {
-    for (int64_t i = 0; i < Len; i++) {
-        out.data[i] = in.data[i] + 1.0f;
-    }
+    std::transform(in.data, in.data + Len, out.data, [](float v) { return v + 1.0f; });
 }
 
 }  // namespace impl
