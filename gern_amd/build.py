@@ -60,10 +60,24 @@ def build_cpp_tests():
             [src, "-L" + HERE, "-lgern", "-lgern_hip", rpath, "-o", exe])
 
 
+def build_examples():
+    """examples/*.c: hosts in plain C99 over the C ABI (examples/bin/)."""
+    edir = os.path.join(ROOT, "examples")
+    bindir = os.path.join(edir, "bin")
+    os.makedirs(bindir, exist_ok=True)
+    rpath = "-Wl,-rpath,$ORIGIN/../../gern_amd:" + os.path.join(ROCM, "lib")
+    for src in sorted(glob.glob(os.path.join(edir, "*.c"))):
+        exe = os.path.join(bindir, os.path.splitext(os.path.basename(src))[0])
+        run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-O2", "-ffp-contract=off",
+             "-I" + os.path.join(ROOT, "include"), src, "-L" + HERE, "-lgern_pipelines", "-lgern", "-lgern_hip", rpath,
+             "-o", exe])
+
+
 def build_all():
     build_native()
     build_gernel_check()
     build_cpp_tests()
+    build_examples()
 
 
 def sanitize_check():

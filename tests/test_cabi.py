@@ -284,3 +284,25 @@ def test_pipelines_use_the_code_object_cache(tmp_path, monkeypatch):
     assert len(list(tmp_path.iterdir())) in (1, 2)
     assert a.source and b.source
     del cold, warm
+
+
+def _c_example(*args):
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "examples", "bin", "blur_c_host")
+    if not os.path.exists(exe):
+        pytest.fail("%s is missing: run `python gern_amd/build.py`" % exe)
+    return subprocess.run([exe] + list(args), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+
+
+def test_c_host_example_builds_the_pipeline_without_a_device():
+    # examples/blur_c_host.c is strict C99 over include/*.h only
+    p = _c_example("--compile-only")
+    assert p.returncode == 0, p.stdout
+    assert "kernel: function_" in p.stdout
+
+
+@pytest.mark.gpu
+def test_c_host_example_runs_bit_exact_on_the_device():
+    p = _c_example()
+    assert p.returncode == 0, p.stdout
+    assert " 0 differ" in p.stdout, p.stdout
