@@ -537,6 +537,14 @@ const char *gern_pipeline_kernel_name(gern_pipeline p) {
 }
 
 int gern_pipeline_destroy(gern_pipeline p) {
+    if (p != nullptr) {
+        // waits for the device, then frees the loaded code objects
+        for (Runner *r : {p->runner.get(), p->exact.get()}) {
+            if (r != nullptr) {
+                r->release();
+            }
+        }
+    }
     delete p;
     return 0;
 }

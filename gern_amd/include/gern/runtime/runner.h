@@ -72,6 +72,12 @@ public:
     void setStream(void *s) {
         stream = s;
     }
+    // Device launches: waits for the device (a kernel of this Runner may still
+    // be running) and unloads the compiled code.  The destructor does NOT do
+    // this, as the reference never closes its dlopen handle either; a caller
+    // that creates Runners over and over calls release() when it is done with
+    // one.  The Runner cannot evaluate afterwards.
+    void release();
 
 private:
     FunctionSignature signature;

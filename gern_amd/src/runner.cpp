@@ -49,6 +49,18 @@ Runner::~Runner() {
     // reference's dlopen handle: kernels may still be in flight.
 }
 
+void Runner::release() {
+    if (module == nullptr) {
+        return;
+    }
+    if (gern_hip_sync() == GERN_HIP_OK) {
+        gern_hip_module_unload(static_cast<gern_hip_module>(module));
+    }  // else: the device is in an error state; leave the module alone
+    module = nullptr;
+    kernel = nullptr;
+    compiled = false;
+}
+
 void Runner::compile(Options config) {
     codegen::GeneratorOptions gen_options;
     gen_options.xcd_remap = config.xcd_remap;

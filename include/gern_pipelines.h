@@ -105,6 +105,8 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
 const char *gern_pipeline_source(gern_pipeline p);
 /* The name expression of the instantiated kernel, e.g. "function_7<252, 8, 3>". */
 const char *gern_pipeline_kernel_name(gern_pipeline p);
+/* Waits for the device (a run may still be in flight), unloads the pipeline's
+ * code objects and frees the handle. */
 int gern_pipeline_destroy(gern_pipeline p);
 
 size_t gern_pipelines_last_error(char *buf, size_t buf_size);

@@ -480,3 +480,30 @@ def test_kernel_loaded_from_the_code_object_cache_runs(gpu, tmp_path, monkeypatc
         torch.cuda.synchronize()
         expect = expect * 3 + 1
         assert np.array_equal(x.cpu().numpy(), expect), attempt
+
+
+def test_destroying_pipelines_frees_their_code_objects(gpu, oracle):
+    # a server that creates and destroys pipelines must not pile up loaded
+    # modules: destroy waits for the device and unloads them
+    import gc
+    import torch
+    x = oracle.normal((8, 1024), 3, 0.0, 2.0)
+    dx = _dev(x)
+    want = oracle.softmax_rows(x)
+
+    def once():
+        sm = gpu.Softmax(1024)
+        out = torch.empty_like(dx)
+        sm(dx, out)          # still in flight when the pipeline goes away
+        del sm
+        gc.collect()
+        torch.cuda.synchronize()
+        assert np.max(np.abs(out.cpu().numpy() - want) / want) < 1e-5
+
+    for _ in range(3):
+        once()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(40):
+        once()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_before - free_after < 32 * 2 ** 20, (free_before, free_after)
