@@ -124,6 +124,29 @@ def test_blur_tiny_values_and_zeros_stay_exact(gpu, oracle):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_blur_on_windows_of_wider_buffers(gpu, oracle):
+    # row pitches larger than the widths (ld_in, ld_out of the C ABI), windows
+    # that start off the 16-byte grid, and a result written into the middle of
+    # a larger buffer whose other elements must stay untouched
+    import torch
+    big = oracle.uniform((90, 700), 21)
+    d_big = _dev(big)
+    for (r0, c0, rows, cols) in ((0, 0, 90, 520), (3, 4, 60, 600), (5, 1, 70, 333), (2, 3, 9, 17)):
+        win = d_big[r0:r0 + rows, c0:c0 + cols]
+        p = gpu.BlurChain("xyx", tile_rows=6)
+        orows, ocols = p.out_shape(rows, cols)
+        canvas = torch.full((orows + 4, ocols + 9), -7.0, dtype=torch.float32, device="cuda")
+        out = canvas[2:2 + orows, 5:5 + ocols]
+        p(win, out)
+        torch.cuda.synchronize()
+        want = oracle.blur_chain(np.ascontiguousarray(big[r0:r0 + rows, c0:c0 + cols]), "xyx")
+        got = canvas.cpu().numpy()
+        assert np.array_equal(got[2:2 + orows, 5:5 + ocols], want), (r0, c0, rows, cols)
+        frame = got.copy()
+        frame[2:2 + orows, 5:5 + ocols] = -7.0
+        assert np.all(frame == -7.0), (r0, c0, rows, cols)
+
+
 # --------------------------------------------------------------- softmax ----
 def _run_softmax(gpu, x, **kw):
     import torch
@@ -154,6 +177,23 @@ def test_softmax_matches_oracle(gpu, oracle, shape, kw):
     got = _run_softmax(gpu, x, **kw)
     want = oracle.softmax_rows(x)
     assert np.max(np.abs(got - want) / want) < 1e-5
+
+
+def test_softmax_on_a_window_of_a_wider_buffer(gpu, oracle):
+    # ld larger than ncol; columns outside the window stay as they were
+    import torch
+    for ncol, ld, c0 in ((1024, 1280, 0), (1000, 1030, 7), (4096, 4100, 4)):
+        x = oracle.normal((19, ld), 13, 0.0, 2.0)
+        dx = _dev(x)
+        dy = torch.full((19, ld), -7.0, dtype=torch.float32, device="cuda")
+        sm = gpu.Softmax(ncol)
+        sm(dx[:, c0:c0 + ncol], dy[:, c0:c0 + ncol])
+        torch.cuda.synchronize()
+        got = dy.cpu().numpy()
+        want = oracle.softmax_rows(np.ascontiguousarray(x[:, c0:c0 + ncol]))
+        assert np.max(np.abs(got[:, c0:c0 + ncol] - want) / want) < 1e-5, (ncol, ld, c0)
+        got[:, c0:c0 + ncol] = -7.0
+        assert np.all(got == -7.0), (ncol, ld, c0)
 
 
 def test_softmax_full_size(gpu, oracle):
