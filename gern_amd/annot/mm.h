@@ -15,10 +15,11 @@ namespace annot {
 class MatrixOperand : public AbstractDataType {
 public:
     enum Element { F32, BF16 };
-    // exact: the caller guarantees what gernels::GlobalView calls EXACT (the
-    // reduction extent is a multiple of the stage depth, 64 for bf16 and 32 for
-    // fp32; rows are 16-byte aligned whole numbers of 16-byte pieces); the
-    // matrix-core gernels then load both operands straight into LDS.
+    // exact: the caller guarantees what gernels::GlobalView calls EXACT (one
+    // dense allocation per matrix; rows of A 16-byte aligned whole numbers of
+    // 16-byte pieces, i.e. a reduction extent that is a multiple of 8 for bf16
+    // and of 4 for fp32; rows of B 4-byte aligned); the matrix-core gernels
+    // then load both operands straight into LDS.
     MatrixOperand(const std::string &name, Element element, bool exact = false)
         : name(name), element(element), exact(exact) {
     }

@@ -420,13 +420,13 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    // whole K stages, 16-byte aligned operands, rows of B in whole 16-byte pieces, and row pitches (K for A, N for B) within the
-    // fast gernel's 32-bit byte offsets; M and N need not be multiples of the tile
-    const int64_t stage = p->kind == gern_pipeline_s::GEMM_BF16 ? 64 : 32;       // K depth of an LDS stage
+    // The matrix-core gernels (gernels/mm.h, mfma_direct / mfma_direct_f32) take every shape whose rows of
+    // A are whole 16-byte pieces (bf16: K % 8 == 0, required above; fp32: K % 4 == 0) with 16-byte aligned A,
+    // and row pitches (K for A, N for B) within their 32-bit byte offsets; partial tiles and a partial last
+    // K stage are theirs too.
     const int64_t piece = p->kind == gern_pipeline_s::GEMM_BF16 ? 8 : 4;         // elements in 16 bytes
     const int64_t max_pitch = int64_t(1) << 20;                                   // gernels/mm.h, kMfmaMaxLd
-    const bool aligned = ((pa | pb) & 15u) == 0;  // 16-byte loads
-    p->last_run_exact = p->exact && aligned && K % stage == 0 && N % piece == 0 && K <= max_pitch && N <= max_pitch;
+    p->last_run_exact = p->exact && (pa & 15u) == 0 && K % piece == 0 && K <= max_pitch && N <= max_pitch;
     if (p->last_run_exact) {
         runner = p->exact.get();
     }

@@ -39,11 +39,13 @@ extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 
 // A window onto a row-major matrix in HBM: at most R x C, of which
 // rows x cols lie inside the matrix.  EXACT is a promise about the matrix the
-// window was cut from, made by the program that declares the operand: its
-// reduction extent (columns of A, rows of B) is a multiple of the LDS stage
-// depth of the matrix-core gernel (64 for bf16, 32 for fp32), its rows start
-// on 16-byte boundaries and hold a whole number of 16-byte pieces.  Windows on the bottom and right edges may still be
-// partial: rows and cols say how much of them exists.
+// window was cut from, made by the program that declares the operand: the
+// matrix is one dense allocation that ends with its last element, the rows of
+// A start on 16-byte boundaries and hold a whole number of 16-byte pieces (its
+// reduction extent is a multiple of 8 for bf16, of 4 for fp32), the rows of B
+// start on 4-byte boundaries, and row pitches stay below kMfmaMaxLd elements.
+// Windows on the bottom and right edges may be partial, and so may the last
+// stage of the reduction: rows and cols say how much of them exists.
 template<int64_t R, int64_t C, typename T, bool EXACT>
 struct GlobalView {
     const T *data;
@@ -254,7 +256,10 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     const int lane = lane_id();
     const int w = wave_in_block();
     const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
-    const int nk = (int)(k_total / kMfmaBK);
+    // A last stage may be partial (its depth `tail` a multiple of 8, as rows of
+    // A are whole 16-byte pieces): its missing part is ZERO in LDS, see issue().
+    const int nk = (int)((k_total + kMfmaBK - 1) / kMfmaBK);
+    const int tail = (int)(k_total % kMfmaBK);
     if (nk == 0 || A.rows <= 0 || B.cols <= 0) {  // workgroup-uniform
         return;
     }
@@ -292,18 +297,28 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         const int chunk_b = (lane % 32) ^ (4 * ((2 * odd + lane / 32) & 3));
         lane_off_b[odd] = ((lane / 32) * (int)B.lda + (chunk_b < last_chunk_b ? chunk_b : last_chunk_b) * 8) * 2;
     }
-    constexpr int kRawBuffer = 0x00020000;  // 32-bit raw buffer descriptor, no swizzle, no bounds beyond num_records
-    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, -1, kRawBuffer);
+    // Raw 32-bit buffer descriptors whose num_records end at the last valid
+    // element of the window: the hardware checks vector + scalar offset of
+    // every dword against it, and a dword past it reads as ZERO (also into
+    // LDS).  That is how K rows of B past the end of a partial last stage, and
+    // the few elements past the end of the last row, become zeros without a
+    // branch; chunks of A past K lie INSIDE the matrix (in the next row), so
+    // the lanes that would fetch them are sent out of range instead.
+    constexpr int kRawBuffer = 0x00020000;
+    constexpr int kOutOfRange = 0x7FFF0000;
+    const __amdgpu_buffer_rsrc_t desc_a =
+        __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, (int)((((int64_t)A.rows - 1) * A.lda + A.cols) * 2), kRawBuffer);
     const int row_bytes_b = (int)B.lda * 2;
-    auto issue = [&](int kt, unsigned char *dst) {
+    auto issue_from = [&](int kt, unsigned char *dst, const int (&off_a)[4]) {
         const int k0 = kt * (int)kMfmaBK;
-        const __amdgpu_buffer_rsrc_t desc_b =
-            __builtin_amdgcn_make_buffer_rsrc((void *)(B.data + (int64_t)k0 * B.lda), 0, -1, kRawBuffer);
+        const int64_t left_b = (((int64_t)B.rows - 1 - k0) * B.lda + B.cols) * 2;  // bytes from this stage's first row to the end
+        const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(B.data + (int64_t)k0 * B.lda), 0, (int)(left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
-                                                     lane_off_a[j], k0 * 2, 0, 0);
+                                                     off_a[j], k0 * 2, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -311,6 +326,20 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b,
                                                      (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)),
                                                      16, lane_off_b[j & 1], 2 * i * row_bytes_b, 0, 0);
+        }
+    };
+    auto issue = [&](int kt, unsigned char *dst) {
+        if (tail != 0 && kt == nk - 1) {  // workgroup-uniform; at most once per call
+            int off_tail[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int row = 8 * (wu * 4 + j) + lane / 8;
+                const int chunk_a = (lane % 8) ^ ((row >> 1) & 7);
+                off_tail[j] = chunk_a * 8 < tail ? lane_off_a[j] : kOutOfRange;
+            }
+            issue_from(kt, dst, off_tail);
+        } else {
+            issue_from(kt, dst, lane_off_a);
         }
     };
 
@@ -700,7 +729,9 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
     const int lane = lane_id();
     const int w = wave_in_block();
     const int64_t k_total = A.cols < B.rows ? A.cols : B.rows;
-    const int nk = (int)(k_total / BK);
+    // A partial last stage (depth `tail`, a multiple of 4) is zero-filled, as in mfma_direct.
+    const int nk = (int)((k_total + BK - 1) / BK);
+    const int tail = (int)(k_total % BK);
     if (nk == 0 || A.rows <= 0 || B.cols <= 0) {  // workgroup-uniform
         return;
     }
@@ -718,20 +749,26 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
         lane_off_a[j] = ((row < last_row_a ? row : last_row_a) * (int)A.lda + chunk * 4) * 4;
     }
     const int lane_off_b = (lane < last_chunk_b ? lane : last_chunk_b) * 16;
+    // Descriptors that end at the last valid element of each window: dwords
+    // past it (K rows of B beyond a partial last stage, the end of the last
+    // row) read as zero; lanes of A past K are sent out of range (mfma_direct).
     constexpr int kRawBuffer = 0x00020000;
-    const __amdgpu_buffer_rsrc_t desc_a = __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, -1, kRawBuffer);
+    constexpr int kOutOfRange = 0x7FFF0000;
+    const __amdgpu_buffer_rsrc_t desc_a =
+        __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, (int)((((int64_t)A.rows - 1) * A.lda + A.cols) * 4), kRawBuffer);
     const int row_bytes_b = (int)B.lda * 4;
     // Wavefront w issues A instructions 4w .. 4w+3 (8 rows each) and B
     // instructions 4w .. 4w+3 (one K row each) of every stage.
-    auto issue = [&](int kt, unsigned char *dst) {
+    auto issue_from = [&](int kt, unsigned char *dst, const int (&off_a)[4]) {
         const int k0 = kt * BK;
-        const __amdgpu_buffer_rsrc_t desc_b =
-            __builtin_amdgcn_make_buffer_rsrc((void *)(B.data + (int64_t)k0 * B.lda), 0, -1, kRawBuffer);
+        const int64_t left_b = (((int64_t)B.rows - 1 - k0) * B.lda + B.cols) * 4;
+        const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(B.data + (int64_t)k0 * B.lda), 0, (int)(left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
-                                                     lane_off_a[j], k0 * 4, 0, 0);
+                                                     off_a[j], k0 * 4, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -739,6 +776,20 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b,
                                                      (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)),
                                                      16, lane_off_b, i * row_bytes_b, 0, 0);
+        }
+    };
+    auto issue = [&](int kt, unsigned char *dst) {
+        if (tail != 0 && kt == nk - 1) {  // workgroup-uniform; at most once per call
+            int off_tail[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int row = 8 * (wu * 4 + j) + lane / 8;
+                const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+                off_tail[j] = chunk * 4 < tail ? lane_off_a[j] : kOutOfRange;
+            }
+            issue_from(kt, dst, off_tail);
+        } else {
+            issue_from(kt, dst, lane_off_a);
         }
     };
 

@@ -72,16 +72,15 @@ int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows,
 
 /* Dense GEMM C += A * B (or C = A * B with GERN_PIPELINE_GEMM_OVERWRITE),
  * row-major, A is M x K, B is K x N, C is M x N fp32.
- * variant 0: fp32 inputs and fp32 arithmetic.  Shapes with K % 32 == 0 and
- *            N % 4 == 0 (any M) and 16-byte aligned A and B run on the fp32
- *            matrix instruction (v_mfma_f32_32x32x2_f32), operands loaded
- *            straight into LDS; other shapes run on vector-ALU FMAs.  Both sum each dot product in
+ * variant 0: fp32 inputs and fp32 arithmetic.  Shapes with K % 4 == 0 (any M
+ *            and N) and a 16-byte aligned A run on the fp32 matrix instruction
+ *            (v_mfma_f32_32x32x2_f32), operands loaded straight into LDS; other
+ *            shapes run on vector-ALU FMAs.  Both sum each dot product in
  *            fp32; the order of the additions differs.
  * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA; needs
- *            K % 8 == 0 and N % 2 == 0, A 16-byte and B 4-byte aligned.
- *            Shapes with K % 64 == 0 and N % 8 == 0 (any M) and 16-byte aligned
- *            A and B take the faster kernel, which loads both operands
- *            straight into LDS.
+ *            K % 8 == 0 and N % 2 == 0, A 16-byte and B 4-byte aligned.  All
+ *            such shapes take the kernel that loads both operands straight
+ *            into LDS (row pitches up to 2^20 elements).
  * Composes Tile(i)(Tile(j)(Reduce(k)(matrix_multiply))) as
  * gernels/mm/kernel_3.cu:61-75 does. */
 int gern_gemm_create(int variant, int flags, gern_pipeline *out);

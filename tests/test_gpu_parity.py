@@ -284,13 +284,16 @@ def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K, general_only):
     assert np.array_equal(_run_gemm(gpu, "bf16", aib, bib, general_only=general_only), ai @ bi)
 
 
-# Shapes with K % 64 == 0 and N % 8 == 0 take the eight-wavefront kernel that
-# loads straight into LDS: one K stage, an odd number of stages, several
-# column and row tiles, a K that spans more than one 4096-deep Reduce step,
-# and partial tiles at the bottom and right edges (one row, one 8-column
-# chunk, all but one).
+# Every shape the bf16 pipeline accepts (K % 8 == 0, N % 2 == 0) takes the
+# eight-wavefront kernel that loads straight into LDS: one K stage, an odd
+# number of stages, several column and row tiles, a K that spans more than one
+# 4096-deep Reduce step, partial tiles at the bottom and right edges (one row,
+# one 8-column chunk, all but one), a partial last K stage (its missing part
+# must read as zero), rows of B off the 16-byte grid (N not a multiple of 8),
+# two columns, and K below one stage.
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (512, 256, 192), (256, 768, 128), (768, 512, 4096 + 4096 + 64),
-                                   (300, 264, 128), (1, 8, 64), (511, 504, 320), (257, 1000, 64)])
+                                   (300, 264, 128), (1, 8, 64), (511, 504, 320), (257, 1000, 64),
+                                   (256, 256, 72), (300, 258, 200), (130, 262, 8), (77, 2, 120), (512, 302, 4096 + 56)])
 @pytest.mark.parametrize("overwrite", [False, True])
 def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     import torch
@@ -320,12 +323,15 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
 
 
-# fp32 shapes with K % 32 == 0 and N % 4 == 0 take the eight-wavefront kernel
-# on the fp32 matrix instruction: one K stage, an odd number of stages, several
-# tiles either way, a K beyond one 4096-deep Reduce step, and partial tiles at
-# the bottom and right edges (one row, one 4-column piece, all but one).
+# fp32 shapes with K % 4 == 0 take the eight-wavefront kernel on the fp32
+# matrix instruction: one K stage, an odd number of stages, several tiles
+# either way, a K beyond one 4096-deep Reduce step, partial tiles at the bottom
+# and right edges (one row, one 4-column piece, all but one), a partial last K
+# stage (its missing part must read as zero), rows of B off the 16-byte grid
+# (N not a multiple of 4), a single column, and K below one stage.
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (512, 256, 96), (256, 768, 64), (512, 512, 4096 + 4096 + 32),
-                                   (300, 260, 128), (1, 4, 32), (511, 508, 160), (257, 1000, 32)])
+                                   (300, 260, 128), (1, 4, 32), (511, 508, 160), (257, 1000, 32),
+                                   (256, 256, 36), (300, 258, 100), (130, 263, 4), (77, 1, 60), (512, 301, 4096 + 28)])
 @pytest.mark.parametrize("overwrite", [False, True])
 def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     import torch
@@ -355,9 +361,9 @@ def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(K)
 
 
-# Shapes the matrix-core fp32 kernel cannot take (K not a multiple of 32, N not
-# a multiple of 4) stay on the vector-ALU kernel.
-@pytest.mark.parametrize("M,N,K", [(256, 256, 48), (256, 258, 64)])
+# The matrix-core fp32 kernel reads rows of A in whole 16-byte pieces: a K
+# that is not a multiple of 4 stays on the vector-ALU kernel.
+@pytest.mark.parametrize("M,N,K", [(256, 256, 50), (130, 258, 63)])
 def test_gemm_f32_other_shapes_keep_the_general_kernel(gpu, oracle, M, N, K):
     import torch
     ai = np.random.RandomState(51).randint(-3, 4, size=(M, K)).astype(np.float32)
