@@ -17,6 +17,7 @@
 #include <cstring>
 #include <cstdlib>
 #include <memory>
+#include <sstream>
 #include <string>
 
 using namespace gern;
@@ -93,11 +94,22 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
             p->source = cg.generate_code(program);
             p->kernel_name = cg.getLaunchPlan().name_expression;
             p->names = cg.getArgumentOrder();
-            const std::string inc = "-I" + packageDir();
+            // the same options the Runner would pass: "-I <dir>" and whatever GERN_PIPELINE_EXTRA_OPTIONS adds
+            std::vector<std::string> words;
+            std::istringstream in(include);
+            for (std::string w; in >> w;) {
+                if (w == "-I" && (in >> w)) {
+                    w = "-I" + w;
+                }
+                words.push_back(w);
+            }
+            std::vector<const char *> opts;
+            for (const auto &w : words) {
+                opts.push_back(w.c_str());
+            }
             const char *names[1] = {p->kernel_name.c_str()};
-            const char *opts[1] = {inc.c_str()};
             size_t size = 0;
-            if (gern_hip_compile_only(p->source.c_str(), names, 1, opts, 1, "gfx950", &size) != 0) {
+            if (gern_hip_compile_only(p->source.c_str(), names, 1, opts.data(), (int)opts.size(), "gfx950", &size) != 0) {
                 std::string msg(gern_hip_last_error(nullptr, 0) + 1, '\0');
                 gern_hip_last_error(msg.data(), msg.size());
                 return fail("Compilation Failed\n" + msg);
