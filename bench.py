@@ -33,7 +33,7 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3
 # WRITE_SIZE counters scaled by the plain-copy calibration kernel below
 # (profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from
 # inside this process; the figure is re-measured whenever the kernel changes.
-BLUR_XYX_8192_TRAFFIC_BYTES = 548746154
+BLUR_XYX_8192_TRAFFIC_BYTES = 548676945
 
 
 def log(*a):
