@@ -224,7 +224,10 @@ def main():
             "data": "synthetic",
             "config": {"workload": "three-stage fused separable blur chain (3-tap x, y, x; weights 1/3), 8192x8192 fp32 "
                                    "uniform[0,1) seed 2, valid-region output 8190x8188, one launch per step",
-                       "schedule": "one wavefront per 6x252 output tile, XCD-aware workgroup order"},
+                       "schedule": "one wavefront per 6x252 output tile, XCD-aware workgroup order",
+                       "protocol": "the reference's: warm-up, then `steps` launches on the same buffers "
+                                   "(roofline.achieved_rotating_buffers: the same launches over four rotating "
+                                   "buffer pairs, which takes the 256 MiB memory-side cache out of the figure)"},
             "roofline": roof,
         }
         if not args.no_cpu:
