@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-kernel hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-rotating] [--only NAME]
 
 A step is one launch of the fused three-stage blur chain (x, y, x; 3 taps of
 weight 1/3) on an 8192 x 8192 fp32 image that is already resident in HBM; the
@@ -33,7 +33,7 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3
 # WRITE_SIZE counters scaled by the plain-copy calibration kernel below
 # (profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from
 # inside this process; the figure is re-measured whenever the kernel changes.
-BLUR_XYX_8192_TRAFFIC_BYTES = 548676945
+BLUR_XYX_8192_TRAFFIC_BYTES = 548743032
 
 
 def log(*a):
@@ -151,6 +151,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-rotating", action="store_true",
+                    help="skip the extra timings over rotating buffers (profiles: keeps one kind of launch per kernel)")
     ap.add_argument("--only", default="", help="run only this workload (blur, softmax, gemm_f32, gemm_bf16, qk_softmax, copy)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -189,26 +191,27 @@ def main():
         roof["kernel_ms_min"] = each[0]
         workloads["blur_xyx_8192"] = {"GB/s": gbs, "ms": wall, "frac_hbm": gbs / HBM_PEAK_GBS}
         log("blur xyx 8192^2: %.1f us/launch  %.0f GB/s  (%.1f%% of HBM peak)" % (wall * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
-        # The same launch over ROTATING buffer pairs: the 256 MiB image is exactly the size of the
-        # memory-side cache, and with streaming stores a launch finds part of its input there when
-        # the previous launch read the same buffer.  Rotating over four pairs takes that away.
-        ring = [(d_in, d_out)] + [(d_in.clone(), torch.zeros_like(d_out)) for _ in range(3)]
-        turn = [0]
+        if not args.no_rotating:
+            # The same launch over ROTATING buffer pairs: the 256 MiB image is exactly the size of the
+            # memory-side cache, and with streaming stores a launch finds part of its input there when
+            # the previous launch read the same buffer.  Rotating over four pairs takes that away.
+            ring = [(d_in, d_out)] + [(d_in.clone(), torch.zeros_like(d_out)) for _ in range(3)]
+            turn = [0]
 
-        def rotating():
-            a, b = ring[turn[0] % len(ring)]
-            turn[0] += 1
-            blur(a, b)
-        wall_r, ev_r = time_launches(rotating, args.warmup, args.steps, torch, gern_amd)
-        workloads["blur_xyx_8192_rotating_buffers"] = {"GB/s": nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
-                                                       "frac_hbm": nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS, "buffer_pairs": len(ring)}
-        log("blur xyx 8192^2 over %d rotating buffer pairs: %.1f us/launch  %.0f GB/s" % (len(ring), ev_r * 1e3, nbytes / (ev_r * 1e-3) / 1e9))
-        # `value`, `achieved` and `frac` follow the reference's own protocol (apps/blur/blur.cu:79-96: warm-up,
-        # then N launches on the SAME buffers); the rotating figure is what HBM alone sustains.
-        roof["achieved_rotating_buffers"] = nbytes / (ev_r * 1e-3) / 1e9
-        roof["frac_rotating_buffers"] = roof["achieved_rotating_buffers"] / HBM_PEAK_GBS
-        roof["kernel_ms_rotating_buffers"] = ev_r
-        del ring
+            def rotating():
+                a, b = ring[turn[0] % len(ring)]
+                turn[0] += 1
+                blur(a, b)
+            wall_r, ev_r = time_launches(rotating, args.warmup, args.steps, torch, gern_amd)
+            workloads["blur_xyx_8192_rotating_buffers"] = {"GB/s": nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
+                                                           "frac_hbm": nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS, "buffer_pairs": len(ring)}
+            log("blur xyx 8192^2 over %d rotating buffer pairs: %.1f us/launch  %.0f GB/s" % (len(ring), ev_r * 1e3, nbytes / (ev_r * 1e-3) / 1e9))
+            # `value`, `achieved` and `frac` follow the reference's own protocol (apps/blur/blur.cu:79-96: warm-up,
+            # then N launches on the SAME buffers); the rotating figure is what HBM alone sustains.
+            roof["achieved_rotating_buffers"] = nbytes / (ev_r * 1e-3) / 1e9
+            roof["frac_rotating_buffers"] = roof["achieved_rotating_buffers"] / HBM_PEAK_GBS
+            roof["kernel_ms_rotating_buffers"] = ev_r
+            del ring
         result = {
             "metric": "fused 3-stage blur (x,y,x) 8192x8192 fp32, algorithmic GB/s",
             "value": gbs,
@@ -246,19 +249,21 @@ def main():
         gbs = 2 * x.nbytes / (ev * 1e-3) / 1e9
         workloads["softmax_8192x4096"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "kernel": sm.kernel_name}
         log("softmax 8192x4096: %.1f us  %.0f GB/s (%.1f%%)" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
-        ring = [(d_x, d_y)] + [(d_x.clone(), torch.zeros_like(d_y)) for _ in range(5)]
-        turn = [0]
+        if not args.no_rotating:
+            ring = [(d_x, d_y)] + [(d_x.clone(), torch.zeros_like(d_y)) for _ in range(5)]
+            turn = [0]
 
-        def rotating_softmax():
-            a, b = ring[turn[0] % len(ring)]
-            turn[0] += 1
-            sm(a, b)
-        wall_r, ev_r = time_launches(rotating_softmax, args.warmup, steps2, torch, gern_amd)
-        workloads["softmax_8192x4096_rotating_buffers"] = {"GB/s": 2 * x.nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
-                                                           "frac_hbm": 2 * x.nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                                                           "buffer_pairs": len(ring)}
-        log("softmax 8192x4096 over %d rotating buffer pairs: %.1f us  %.0f GB/s" % (len(ring), ev_r * 1e3, 2 * x.nbytes / (ev_r * 1e-3) / 1e9))
-        del d_x, d_y, ring
+            def rotating_softmax():
+                a, b = ring[turn[0] % len(ring)]
+                turn[0] += 1
+                sm(a, b)
+            wall_r, ev_r = time_launches(rotating_softmax, args.warmup, steps2, torch, gern_amd)
+            workloads["softmax_8192x4096_rotating_buffers"] = {"GB/s": 2 * x.nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
+                                                               "frac_hbm": 2 * x.nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                                               "buffer_pairs": len(ring)}
+            log("softmax 8192x4096 over %d rotating buffer pairs: %.1f us  %.0f GB/s" % (len(ring), ev_r * 1e3, 2 * x.nbytes / (ev_r * 1e-3) / 1e9))
+            del ring
+        del d_x, d_y
 
     # ---- config 4: GEMM 4096^3 ---------------------------------------------
     for variant, peak in (("f32", FP32_VECTOR_PEAK_TFLOPS), ("bf16", MFMA_BF16_PEAK_TFLOPS)):
@@ -316,11 +321,12 @@ def main():
                                                                      "gern_copy_f4_streaming")
         log("copy 256 MiB, streaming stores: %.1f us  %.0f GB/s" % (workloads["copy_256MiB_streaming_stores"]["ms"] * 1e3,
                                                                    workloads["copy_256MiB_streaming_stores"]["GB/s"]))
-        # 1 GiB: far beyond the 256 MiB memory-side cache, i.e. what HBM itself streams
-        workloads["copy_1GiB_streaming_stores"] = copy_calibration(torch, gern_amd, args.warmup, max(10, steps2 // 2),
-                                                                   "gern_copy_f4_streaming", 1 << 30)
-        log("copy 1 GiB, streaming stores: %.1f us  %.0f GB/s" % (workloads["copy_1GiB_streaming_stores"]["ms"] * 1e3,
-                                                                 workloads["copy_1GiB_streaming_stores"]["GB/s"]))
+        if not args.no_rotating:
+            # 1 GiB: far beyond the 256 MiB memory-side cache, i.e. what HBM itself streams
+            workloads["copy_1GiB_streaming_stores"] = copy_calibration(torch, gern_amd, args.warmup, max(10, steps2 // 2),
+                                                                       "gern_copy_f4_streaming", 1 << 30)
+            log("copy 1 GiB, streaming stores: %.1f us  %.0f GB/s" % (workloads["copy_1GiB_streaming_stores"]["ms"] * 1e3,
+                                                                     workloads["copy_1GiB_streaming_stores"]["GB/s"]))
 
     if result is None:
         result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "", "n_gpus": 1,
