@@ -161,6 +161,8 @@ def main():
     import numpy as np
     import torch
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()  # builds only in a fresh checkout
     import gern_amd
     from gern_amd import inputs
 

@@ -11,6 +11,9 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # a fresh checkout has no native libraries or test programs yet: build them once
+    import __graft_entry__
+    __graft_entry__.ensure_built()
 
 
 @pytest.fixture(scope="session")
