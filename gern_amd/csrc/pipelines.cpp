@@ -58,7 +58,10 @@ AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
 struct gern_pipeline_s {
     enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
-    std::unique_ptr<Runner> exact;   // GEMM: the direct-to-LDS matrix-core kernel (whole K stages, 16-byte row pieces)
+    std::unique_ptr<Runner> exact;   // GEMM: the direct-to-LDS matrix-core kernel (rows of A in whole 16-byte pieces)
+    std::unique_ptr<Runner> tail;    // fp32 GEMM in overwrite mode: C += of the last K % 4 columns, made on first use
+    bool accumulate = true;          // GEMM: C += A * B (false: C = A * B)
+    int create_flags = 0;
     std::string source;
     std::string kernel_name;
     std::string exact_source, exact_kernel_name;
@@ -354,6 +357,8 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
     auto p = std::make_unique<gern_pipeline_s>();
     p->kind = variant == 1 ? gern_pipeline_s::GEMM_BF16 : gern_pipeline_s::GEMM_F32;
     const bool accumulate = !(flags & GERN_PIPELINE_GEMM_OVERWRITE);
+    p->accumulate = accumulate;
+    p->create_flags = flags;
     try {
         const bool bf16 = variant == 1;
         const auto element = bf16 ? annot::MatrixOperand::BF16 : annot::MatrixOperand::F32;
@@ -432,19 +437,47 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
     hip::MatrixF32 c{C, M, N, N};
     int64_t k_dim = K;
     Runner *runner = p->runner.get();
-    // The matrix-core gernels (gernels/mm.h, mfma_direct / mfma_direct_f32) take every shape whose rows of
-    // A are whole 16-byte pieces (bf16: K % 8 == 0, required above; fp32: K % 4 == 0) with 16-byte aligned A,
-    // and row pitches (K for A, N for B) within their 32-bit byte offsets; partial tiles and a partial last
-    // K stage are theirs too.
-    const int64_t piece = p->kind == gern_pipeline_s::GEMM_BF16 ? 8 : 4;         // elements in 16 bytes
-    const int64_t max_pitch = int64_t(1) << 20;                                   // gernels/mm.h, kMfmaMaxLd
-    p->last_run_exact = p->exact && (pa & 15u) == 0 && K % piece == 0 && K <= max_pitch && N <= max_pitch;
-    if (p->last_run_exact) {
-        runner = p->exact.get();
-    }
+    // The matrix-core gernels (gernels/mm.h, mfma_direct / mfma_direct_f32) read rows of A in whole 16-byte
+    // pieces (bf16: K % 8 == 0, required above) with a 16-byte aligned A, and need row pitches (K for A, N for
+    // B) within their 32-bit byte offsets; partial tiles and a partial last K stage are theirs too.  An fp32
+    // product whose K is not a multiple of 4 is split: the first K - K % 4 columns of A (rows of B) go to the
+    // matrix cores, the last one to three are added by the vector-ALU kernel in a second launch.
+    const bool fp32 = p->kind == gern_pipeline_s::GEMM_F32;
+    const int64_t k_main = fp32 ? K - K % 4 : K;
+    const int64_t max_pitch = int64_t(1) << 20;  // gernels/mm.h, kMfmaMaxLd
+    p->last_run_exact = p->exact && (pa & 15u) == 0 && k_main > 0 && K <= max_pitch && N <= max_pitch;
     try {
-        runner->setStream(stream);
-        runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
+        if (!p->last_run_exact) {
+            runner->setStream(stream);
+            runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
+            return 0;
+        }
+        a.col = k_main;
+        b.row = k_main;
+        k_dim = k_main;
+        p->exact->setStream(stream);
+        p->exact->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"k_dim", &k_dim}});
+        if (k_main < K) {
+            Runner *rest = p->runner.get();  // accumulates unless the pipeline overwrites C
+            if (!p->accumulate) {
+                if (!p->tail) {
+                    gern_pipeline_s made;
+                    if (finish(&made,
+                               gemmProgram(annot::MatrixOperand::F32, false, annot::MatrixAccumulator::FMA, true, 128, 128, 256,
+                                           2 * 2 * 16 * 132 * 4),
+                               p->create_flags | GERN_PIPELINE_NO_XCD_REMAP) != 0) {
+                        return 1;
+                    }
+                    p->tail = std::move(made.runner);
+                }
+                rest = p->tail.get();
+            }
+            hip::MatrixF32 a2{a.data + k_main, M, K - k_main, K};
+            hip::MatrixF32 b2{b.data + k_main * N, K - k_main, N, N};
+            int64_t k_rest = K - k_main;
+            rest->setStream(stream);
+            rest->evaluate({{"A", &a2}, {"B", &b2}, {"C", &c}, {"k_dim", &k_rest}});
+        }
     } catch (const std::exception &e) {
         return fail(e.what());
     }
@@ -551,7 +584,7 @@ const char *gern_pipeline_kernel_name(gern_pipeline p) {
 int gern_pipeline_destroy(gern_pipeline p) {
     if (p != nullptr) {
         // waits for the device, then frees the loaded code objects
-        for (Runner *r : {p->runner.get(), p->exact.get()}) {
+        for (Runner *r : {p->runner.get(), p->exact.get(), p->tail.get()}) {
             if (r != nullptr) {
                 r->release();
             }

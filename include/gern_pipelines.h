@@ -72,11 +72,13 @@ int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows,
 
 /* Dense GEMM C += A * B (or C = A * B with GERN_PIPELINE_GEMM_OVERWRITE),
  * row-major, A is M x K, B is K x N, C is M x N fp32.
- * variant 0: fp32 inputs and fp32 arithmetic.  Shapes with K % 4 == 0 (any M
- *            and N) and a 16-byte aligned A run on the fp32 matrix instruction
- *            (v_mfma_f32_32x32x2_f32), operands loaded straight into LDS; other
- *            shapes run on vector-ALU FMAs.  Both sum each dot product in
- *            fp32; the order of the additions differs.
+ * variant 0: fp32 inputs and fp32 arithmetic.  With a 16-byte aligned A the
+ *            product runs on the fp32 matrix instruction
+ *            (v_mfma_f32_32x32x2_f32), operands loaded straight into LDS; when
+ *            K is not a multiple of 4, the last K % 4 columns of A are added by
+ *            a second launch of the vector-ALU kernel, which also takes K < 4
+ *            and unaligned A.  Both sum each dot product in fp32; the order of
+ *            the additions differs.
  * variant 1: bf16 inputs (bit patterns), fp32 accumulation on MFMA; needs
  *            K % 8 == 0 and N % 2 == 0, A 16-byte and B 4-byte aligned.  All
  *            such shapes take the kernel that loads both operands straight

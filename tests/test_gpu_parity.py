@@ -323,7 +323,7 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
 
 
-# fp32 shapes with K % 4 == 0 take the eight-wavefront kernel on the fp32
+# fp32 shapes with K >= 4 take the eight-wavefront kernel on the fp32
 # matrix instruction: one K stage, an odd number of stages, several tiles
 # either way, a K beyond one 4096-deep Reduce step, partial tiles at the bottom
 # and right edges (one row, one 4-column piece, all but one), a partial last K
@@ -331,7 +331,10 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
 # (N not a multiple of 4), a single column, and K below one stage.
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (512, 256, 96), (256, 768, 64), (512, 512, 4096 + 4096 + 32),
                                    (300, 260, 128), (1, 4, 32), (511, 508, 160), (257, 1000, 32),
-                                   (256, 256, 36), (300, 258, 100), (130, 263, 4), (77, 1, 60), (512, 301, 4096 + 28)])
+                                   (256, 256, 36), (300, 258, 100), (130, 263, 4), (77, 1, 60), (512, 301, 4096 + 28),
+                                   # K not a multiple of 4: the last one to three columns of A are added by a
+                                   # second launch of the vector-ALU kernel
+                                   (256, 256, 50), (130, 258, 63), (300, 301, 4096 + 33), (65, 12, 5)])
 @pytest.mark.parametrize("overwrite", [False, True])
 def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     import torch
@@ -361,9 +364,9 @@ def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(K)
 
 
-# The matrix-core fp32 kernel reads rows of A in whole 16-byte pieces: a K
-# that is not a multiple of 4 stays on the vector-ALU kernel.
-@pytest.mark.parametrize("M,N,K", [(256, 256, 50), (130, 258, 63)])
+# The matrix-core fp32 kernel reads rows of A in whole 16-byte pieces; a K
+# below 4 has none and stays on the vector-ALU kernel.
+@pytest.mark.parametrize("M,N,K", [(256, 256, 3), (7, 5, 2)])
 def test_gemm_f32_other_shapes_keep_the_general_kernel(gpu, oracle, M, N, K):
     import torch
     ai = np.random.RandomState(51).randint(-3, 4, size=(M, K)).astype(np.float32)
