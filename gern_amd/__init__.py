@@ -220,7 +220,7 @@ class Softmax(_Pipeline):
 
 class Gemm(_Pipeline):
     """C += A @ B (or C = A @ B with overwrite=True).  variant "f32" or "bf16"
-    (fp32 accumulate); general_only=True keeps shapes that the whole-stage
+    (fp32 accumulate); general_only=True keeps shapes that the direct-to-LDS
     matrix-core kernels could take on the kernel for every shape."""
 
     def __init__(self, variant="f32", overwrite=False, general_only=False, flags=0):

@@ -381,7 +381,7 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
                                            2 * 2 * 16 * 132 * 4),
                                flags);
         if (rc == 0 && !(flags & GERN_PIPELINE_GEMM_GENERAL_ONLY)) {
-            // The same program on data structures that promise whole K stages:
+            // The same program on data structures that promise rows of A in whole 16-byte pieces:
             // eight wavefronts, 256x256 tile on the matrix cores (also for fp32),
             // loads straight into LDS.  Those gernels keep their two stages in
             // static LDS (gernels/mm.h, mfma_direct / mfma_direct_f32): no dynamic LDS.

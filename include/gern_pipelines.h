@@ -40,7 +40,7 @@ enum {
     GERN_PIPELINE_GEMM_OVERWRITE = 4,
     /* GEMM only: build and run only the kernel that takes every shape (fp32:
      * vector-ALU FMAs; bf16: the four-wavefront kernel that stages through
-     * registers), also for shapes the whole-stage kernels could take. */
+     * registers), also for shapes the direct-to-LDS matrix-core kernels take. */
     GERN_PIPELINE_GEMM_GENERAL_ONLY = 8
 };
 

@@ -175,7 +175,7 @@ def test_whole_tile_gemm_reads_one_stage_while_the_other_fills(tmp_path, variant
 
 @pytest.mark.parametrize("variant", ["f32", "bf16"])
 def test_gemm_general_only_builds_one_kernel(tmp_path, variant):
-    # without the flag a GEMM pipeline holds two kernels (the whole-stage
+    # without the flag a GEMM pipeline holds two kernels (the direct-to-LDS
     # matrix-core one with 512 threads, and the one for every shape); with it,
     # only the latter
     os.environ["GERN_HIP_KEEP_DIR"] = str(tmp_path)

@@ -88,7 +88,7 @@ def test_gemm_random_shapes(gpu, oracle, variant):
         if variant == "bf16":
             N = max(2, N // 2 * 2)
             K = max(8, K // 8 * 8)
-            if case % 2 == 0:                 # the direct-to-LDS kernel: K % 64 == 0, N % 8 == 0
+            if case % 2 == 0:                 # whole K stages and 16-byte rows of B
                 K = max(64, K // 64 * 64)
                 N = max(8, N // 8 * 8)
         overwrite = bool(case % 3 == 0)
