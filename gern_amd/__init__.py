@@ -19,6 +19,7 @@ COMPILE_ONLY = 1
 NO_XCD_REMAP = 2
 GEMM_OVERWRITE = 4
 GEMM_GENERAL_ONLY = 8
+BLUR_PLAIN_STORES = 16
 
 _libs = None
 
@@ -181,11 +182,12 @@ class _Pipeline:
 class BlurChain(_Pipeline):
     """Fused separable box blur, e.g. BlurChain("xyx")."""
 
-    def __init__(self, pattern, stride=3, tile_rows=8, tile_cols=None, waves_per_block=1, flags=0):
+    def __init__(self, pattern, stride=3, tile_rows=4, tile_cols=None, waves_per_block=1, flags=0):
         super().__init__()
         nx = pattern.count("x")
         if tile_cols is None:
-            tile_cols = (256 - nx * (stride - 1)) // 4 * 4
+            # the widest tile that writes line-aligned windows (include/gern_pipelines.h)
+            tile_cols = (256 - 28 - nx * (stride - 1)) // 32 * 32
         self.pattern, self.stride = pattern, stride
         self.nx, self.ny = nx, pattern.count("y")
         _check(pipelines_lib().gern_blur_chain_create(pattern.encode(), stride, tile_rows, tile_cols,

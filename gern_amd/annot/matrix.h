@@ -40,15 +40,23 @@ namespace annot {
 //   role OUTPUT : query only names the tile; the producer overwrites it and
 //                 insert stores it (clipped to the matrix)
 //   role TEMP   : never in memory; allocate makes a register tile
+//   roles INPUT_WIDE / OUTPUT_LINES : a pair for a grid of one-chunk tiles
+//                 whose width is a multiple of 32 columns: insert moves each
+//                 tile's window to whole 128-byte lines of the result, and the
+//                 query of the input loads the lanes past the tile's width that
+//                 such a window needs (gernels/wave_tile.h, store_wave_lines)
 class MatrixF32 : public TableADT {
 public:
-    enum Role { INPUT, OUTPUT, ACCUMULATE, TEMP };
+    enum Role { INPUT, OUTPUT, ACCUMULATE, TEMP, INPUT_WIDE, OUTPUT_LINES };
 
     MatrixF32(const std::string &name, Role role)
         : TableADT(name, role == TEMP ? "auto" : "gernels::MatrixF32"), role(role) {
         fields = {x, y, row, col};
-        setCalls("gernels::allocate_wave_tile", role == OUTPUT ? "template view_wave" : "template load_wave", "store_wave");
-        query_is_written_back = role == OUTPUT || role == ACCUMULATE;
+        const bool written = role == OUTPUT || role == OUTPUT_LINES;
+        setCalls("gernels::allocate_wave_tile",
+                 written ? "template view_wave" : role == INPUT_WIDE ? "template load_wave_wide" : "template load_wave",
+                 role == OUTPUT_LINES ? "store_wave_lines" : "store_wave");
+        query_is_written_back = written || role == ACCUMULATE;
         temporaries_are_freed = false;
     }
     // Launch dimensions are computed on the host from the caller's object.

@@ -168,8 +168,13 @@ int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_row
     p->ny = ny;
     p->stride = stride;
     try {
-        auto input = f32("input", annot::MatrixF32::INPUT);
-        auto output = f32("output", annot::MatrixF32::OUTPUT);
+        // Tiles a whole number of 128-byte lines wide that leave 28 columns
+        // of the wavefront's 256 free write line-aligned windows of the result
+        // (gernels/wave_tile.h, store_wave_lines).
+        const bool lines = tile_cols % 32 == 0 && tile_cols + 28 + nx * (stride - 1) <= 256 &&
+                           !(flags & GERN_PIPELINE_BLUR_PLAIN_STORES);
+        auto input = f32("input", lines ? annot::MatrixF32::INPUT_WIDE : annot::MatrixF32::INPUT);
+        auto output = f32("output", lines ? annot::MatrixF32::OUTPUT_LINES : annot::MatrixF32::OUTPUT);
         Variable stride_v("stride"), row("row"), col("col"), col_block("col_block"), wave("wave");
         std::vector<Composable> stages;
         AbstractDataTypePtr prev = input;

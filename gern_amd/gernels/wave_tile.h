@@ -175,6 +175,25 @@ struct MatrixF32 {
         return t;
     }
 
+    // The same tile with EVERY column of its 256-column chunks that lies
+    // inside the matrix, also those past the tile's logical width C.  A chain
+    // of lane-wise stages then produces valid results in those lanes too, which
+    // is what store_wave_lines needs to move its window to cache-line boundaries.
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ WaveTile<R, C> load_wave_wide(int64_t x, int64_t y) const {
+        constexpr int64_t W = WaveTile<R, C>::chunks * kWaveCols;
+        const WaveTile<R, W> t = load_wave<R, W>(x, y);
+        WaveTile<R, C> out;
+#pragma unroll
+        for (int64_t r = 0; r < R; r++) {
+#pragma unroll
+            for (int64_t k = 0; k < WaveTile<R, C>::chunks; k++) {
+                out.v[r][k] = t.v[r][k];
+            }
+        }
+        return out;
+    }
+
     // An output tile: nothing is read, the producer overwrites every element.
     template<int64_t R, int64_t C>
     __device__ __forceinline__ WaveTile<R, C> view_wave(int64_t, int64_t) const {
@@ -211,6 +230,52 @@ struct MatrixF32 {
                     if (lc + 2 < C && cc + 2 < col) p[lc + 2] = val.z;
                     if (lc + 3 < C && cc + 3 < col) p[lc + 3] = val.w;
                 }
+            }
+        }
+    }
+
+    // store_wave for a row of tiles that are C columns apart (C a multiple of
+    // 32, one chunk), with every tile's window moved to whole 128-byte lines:
+    // in row r the tile at column y writes from the first line boundary at or
+    // after y (from column 0 when y == 0) up to the first line boundary at or
+    // after y + C (up to the end of the row for the last tile).  Neighbouring
+    // tiles agree on each boundary, so every element is still written exactly
+    // once, and no line is shared between two wavefronts except the one that
+    // holds the end of one row and the start of the next.  A window starts up
+    // to 28 columns past y, so the lanes past C must hold valid results
+    // (load_wave_wide, and C + 28 + the halo of the chain <= 256).  Partial
+    // lines cost a read-modify-write at the memory side: on an 8192 x 8192
+    // image whose result rows are 8188 floats apart, line-aligned windows take
+    // the x,y,x chain from 101 to 95 us when its buffers come from HBM.
+    // Rows that do not start on a 16-byte boundary keep the plain window.
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ void store_wave_lines(int64_t x, int64_t y, const WaveTile<R, C> &t) const {
+        static_assert(WaveTile<R, C>::chunks == 1 && C % 32 == 0, "line-aligned windows: one chunk, whole lines per tile");
+        const int lane = lane_id();
+        const int64_t cc = y + 4 * lane;
+#pragma unroll
+        for (int64_t r = 0; r < R; r++) {
+            const int64_t rr = x + r;
+            if (rr >= row) {
+                continue;
+            }
+            float *p = data + rr * lda;
+            const uint64_t a0 = (uint64_t)(p + y), a1 = (uint64_t)(p + y + C);
+            const bool vec_ok = (a0 & 15u) == 0;  // wave-uniform
+            int64_t lo = y, hi = y + C;
+            if (vec_ok) {
+                lo = y == 0 ? 0 : y + (int64_t)(((128 - (a0 & 127u)) & 127u) / 4);
+                hi = y + C + (int64_t)(((128 - (a1 & 127u)) & 127u) / 4);
+            }
+            hi = hi < col ? hi : col;
+            const float4 val = t.v[r][0];
+            if (vec_ok && cc >= lo && cc + 3 < hi) {
+                store_streaming(p + cc, val);
+            } else {
+                if (cc + 0 >= lo && cc + 0 < hi) p[cc + 0] = val.x;
+                if (cc + 1 >= lo && cc + 1 < hi) p[cc + 1] = val.y;
+                if (cc + 2 >= lo && cc + 2 < hi) p[cc + 2] = val.z;
+                if (cc + 3 >= lo && cc + 3 < hi) p[cc + 3] = val.w;
             }
         }
     }

@@ -41,7 +41,10 @@ enum {
     /* GEMM only: build and run only the kernel that takes every shape (fp32:
      * vector-ALU FMAs; bf16: the four-wavefront kernel that stages through
      * registers), also for shapes the direct-to-LDS matrix-core kernels take. */
-    GERN_PIPELINE_GEMM_GENERAL_ONLY = 8
+    GERN_PIPELINE_GEMM_GENERAL_ONLY = 8,
+    /* Blur only: every tile stores exactly its own tile_cols columns, also
+     * when tile_cols would allow windows moved to whole 128-byte lines. */
+    GERN_PIPELINE_BLUR_PLAIN_STORES = 16
 };
 
 /* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
@@ -50,7 +53,11 @@ enum {
  * produces the valid region only.  One wavefront produces one
  * tile_rows x tile_cols output tile; tile_cols + (#x stages)*(stride-1) must
  * not exceed 256.  waves_per_block wavefronts (side by side along the
- * columns) form a workgroup.
+ * columns) form a workgroup.  When tile_cols is a multiple of 32 and
+ * tile_cols + 28 + (#x stages)*(stride-1) <= 256 (224 for up to two 3-tap x
+ * stages), each wavefront moves the columns it stores, row by row, to whole
+ * 128-byte lines of the result: the same elements are written, each once, by
+ * possibly a neighbouring wavefront, and no partial line reaches memory.
  * Composes what apps/blur/blur.cpp:31-73 composes (there: blur_x, blur_y). */
 int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_rows, int64_t tile_cols,
                            int waves_per_block, int flags, gern_pipeline *out);

@@ -34,16 +34,33 @@ def test_pipeline_abi_exports_every_declared_symbol():
 
 
 def test_blur_chain_generates_fused_kernel_with_inferred_halos():
-    p = gern_amd.BlurChain("xyx", tile_rows=8, flags=gern_amd.COMPILE_ONLY)
+    p = gern_amd.BlurChain("xyx", tile_rows=8, tile_cols=252, flags=gern_amd.COMPILE_ONLY)
     src = p.source
     assert p.kernel_name.endswith("<252, 8, 3, 64>")
     assert src.count("__global__") == 1 and "__launch_bounds__(64)" in src
     # input tile: (row + 2) x (col + 4); first temporary (row + 2) x (col + 2)
     assert "load_wave<((row + stride) - 1), ((((col + stride) - 1) + stride) - 1)>" in src
+    assert "store_wave(" in src
     assert "allocate_wave_tile<((row + stride) - 1), ((col + stride) - 1)>" in src
     assert "allocate_wave_tile<row, ((col + stride) - 1)>" in src
     assert src.index("blur_x<stride>") < src.index("blur_y<stride>") < src.rindex("blur_x<stride>")
     assert "gern_block_x" in src  # XCD-aware workgroup order
+
+
+def test_blur_chain_line_aligned_windows_by_default():
+    # tiles of 224 columns (seven 128-byte lines) leave the 28 spare columns that
+    # windows moved to line boundaries need: the default schedule
+    p = gern_amd.BlurChain("xyx", tile_rows=6, flags=gern_amd.COMPILE_ONLY)
+    assert p.kernel_name.endswith("<224, 6, 3, 64>")
+    assert "load_wave_wide<((row + stride) - 1), ((((col + stride) - 1) + stride) - 1)>" in p.source
+    assert "store_wave_lines(" in p.source
+    # three x stages of five taps leave room for 192 columns only
+    assert gern_amd.BlurChain("xxx", stride=5, flags=gern_amd.COMPILE_ONLY).kernel_name.split("<")[1].startswith("192,")
+    # asked not to, or with a tile that is not whole lines wide, a tile stores its own columns
+    for kw in ({"flags": gern_amd.COMPILE_ONLY | gern_amd.BLUR_PLAIN_STORES}, {"tile_cols": 228, "flags": gern_amd.COMPILE_ONLY},
+               {"tile_cols": 240, "flags": gern_amd.COMPILE_ONLY}):
+        src = gern_amd.BlurChain("xyx", **kw).source
+        assert "store_wave(" in src and "store_wave_lines" not in src and "load_wave_wide" not in src
 
 
 def test_blur_chain_wavefront_mapping_and_plain_order():

@@ -49,6 +49,13 @@ def test_blur_golden_vectors(gpu, golden, name, pattern):
     ((300, 700), "yxy", {"tile_rows": 8}),
     ((64, 64), "x", {}),
     ((64, 64), "y", {"tile_cols": 128}),
+    # the widest tile (stores its own 252 columns) and the default one (224 columns, windows moved to whole lines)
+    ((1024, 1024), "xyx", {"tile_rows": 6, "tile_cols": 252}),
+    ((100, 1500), "xyx", {"tile_rows": 6, "flags": 16}),        # GERN_PIPELINE_BLUR_PLAIN_STORES
+    ((100, 1500), "xyx", {"tile_rows": 5, "tile_cols": 64}),    # narrow line-aligned tiles, result rows 1496 floats apart
+    ((61, 2047), "xy", {"tile_rows": 3, "tile_cols": 192, "waves_per_block": 2}),  # result rows 2045 floats apart: mostly unaligned
+    ((40, 228), "xyx", {"tile_rows": 8}),                       # exactly one tile of 224 columns
+    ((40, 229), "xyx", {"tile_rows": 8}),                       # one column into the second tile
 ])
 def test_blur_matches_oracle_bit_exact(gpu, oracle, shape, pattern, kw):
     img = oracle.uniform(shape, 7)
@@ -67,18 +74,19 @@ def test_blur_reference_closed_form_on_gpu(gpu, oracle):
 def test_blur_full_size_three_stage(gpu, oracle):
     import torch
     img = oracle.uniform((8192, 8192), 2)
+    # the schedule bench.py times: one wavefront per 4 x 224 output tile, line-aligned store windows
     got = _run_blur(gpu, img, "xyx", tile_rows=4)
     assert got.shape == (8190, 8188)
-    # exact against the oracle on three bands (top, an interior tile seam, bottom)
-    for r0 in (0, 4093, 8190 - 64):
+    # exact against the oracle on four bands (top, two interior tile seams, bottom)
+    for r0 in (0, 4093, 4 * 1100 - 3, 8190 - 64):
         want = oracle.blur_chain(img[r0:r0 + 66], "xyx")
         assert np.array_equal(got[r0:r0 + 64], want)
     # size-independent properties over the whole image: a constant image is a
     # fixed point, and the schedule does not change a single bit
     const = np.full((8192, 8192), 0.375, dtype=np.float32)
     assert np.all(_run_blur(gpu, const, "xyx", tile_rows=4) == np.float32(0.375))
-    again = _run_blur(gpu, img, "xyx", tile_rows=8, waves_per_block=4)
-    assert np.array_equal(got, again)
+    for kw in ({"tile_rows": 6, "tile_cols": 252}, {"tile_rows": 8, "waves_per_block": 4}):
+        assert np.array_equal(got, _run_blur(gpu, img, "xyx", **kw)), kw
     del torch
 
 
@@ -131,20 +139,23 @@ def test_blur_on_windows_of_wider_buffers(gpu, oracle):
     import torch
     big = oracle.uniform((90, 700), 21)
     d_big = _dev(big)
-    for (r0, c0, rows, cols) in ((0, 0, 90, 520), (3, 4, 60, 600), (5, 1, 70, 333), (2, 3, 9, 17)):
-        win = d_big[r0:r0 + rows, c0:c0 + cols]
-        p = gpu.BlurChain("xyx", tile_rows=6)
-        orows, ocols = p.out_shape(rows, cols)
-        canvas = torch.full((orows + 4, ocols + 9), -7.0, dtype=torch.float32, device="cuda")
-        out = canvas[2:2 + orows, 5:5 + ocols]
-        p(win, out)
-        torch.cuda.synchronize()
-        want = oracle.blur_chain(np.ascontiguousarray(big[r0:r0 + rows, c0:c0 + cols]), "xyx")
-        got = canvas.cpu().numpy()
-        assert np.array_equal(got[2:2 + orows, 5:5 + ocols], want), (r0, c0, rows, cols)
-        frame = got.copy()
-        frame[2:2 + orows, 5:5 + ocols] = -7.0
-        assert np.all(frame == -7.0), (r0, c0, rows, cols)
+    # result pitches: odd (most rows start off the 16-byte grid and keep their own columns) and a
+    # multiple of four floats (every row moves its windows to whole 128-byte lines)
+    for (pad, off) in ((9, 5), (12, 8)):
+        for (r0, c0, rows, cols) in ((0, 0, 90, 520), (3, 4, 60, 600), (5, 1, 70, 333), (2, 3, 9, 17)):
+            win = d_big[r0:r0 + rows, c0:c0 + cols]
+            p = gpu.BlurChain("xyx", tile_rows=6)
+            orows, ocols = p.out_shape(rows, cols)
+            canvas = torch.full((orows + 4, ocols + pad), -7.0, dtype=torch.float32, device="cuda")
+            out = canvas[2:2 + orows, off:off + ocols]
+            p(win, out)
+            torch.cuda.synchronize()
+            want = oracle.blur_chain(np.ascontiguousarray(big[r0:r0 + rows, c0:c0 + cols]), "xyx")
+            got = canvas.cpu().numpy()
+            assert np.array_equal(got[2:2 + orows, off:off + ocols], want), (pad, off, r0, c0, rows, cols)
+            frame = got.copy()
+            frame[2:2 + orows, off:off + ocols] = -7.0
+            assert np.all(frame == -7.0), (pad, off, r0, c0, rows, cols)
 
 
 # --------------------------------------------------------------- softmax ----
@@ -404,9 +415,14 @@ def test_gemm_full_size(gpu, oracle, variant, tol):
         A, av = oracle.to_bf16(A)
         B, bv = oracle.to_bf16(B)
     got = _run_gemm(gpu, variant, A, B)
-    rows = (1000, 1002)
-    want = (oracle.gemm_bf16(A, B, rows=rows) if variant == "bf16" else oracle.gemm_f32(A, B, rows=rows))[rows[0]:rows[1]]
-    assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < tol
+    # 64 whole rows against the oracle (every column, the last ones included):
+    # the first and last rows of the first and last 256-row tiles, both sides of
+    # two tile seams, of a wavefront seam and of an MFMA-tile seam inside a tile
+    bands = ((0, 8), (248, 264), (1000, 1002), (1148, 1156), (2032, 2048), (2300, 2306), (4088, 4096))
+    assert sum(b - a for a, b in bands) == 64
+    for rows in bands:
+        want = (oracle.gemm_bf16(A, B, rows=rows) if variant == "bf16" else oracle.gemm_f32(A, B, rows=rows))[rows[0]:rows[1]]
+        assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < tol, rows
     # Freivalds-style check of the whole product: C r == A (B r) in fp64
     r = np.random.RandomState(9).randint(0, 2, size=(N,)).astype(np.float64)
     a64 = av.astype(np.float64) if variant == "bf16" else A.astype(np.float64)
@@ -485,14 +501,41 @@ def test_qk_softmax_full_size(gpu, oracle):
     kb, kv = oracle.to_bf16(oracle.normal((N, D), 6))
     scale = np.float32(1.0 / np.sqrt(D))
     got = _run_qk(gpu, qb, kb, scale, 4096)
+    # against the oracle (the CPU pipeline: sequential fp32 sums, expf): first and last row blocks, a seam
     for r0 in (0, 2049, 4096 - 16):
         want = oracle.qk_softmax(qb, kb, scale, rows=(r0, r0 + 16))[r0:r0 + 16]
         assert np.max(np.abs(got[r0:r0 + 16] - want) / want) < 1e-2
     assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
-    # the softmax stage alone, fed identical fp32 logits, is held to 1e-5:
-    # recover the logits' ordering from the result and compare argmax per row
-    logits = (qv[:64].astype(np.float64) @ kv.T.astype(np.float64)) * float(scale)
-    assert np.all(got[:64].argmax(axis=1) == logits.argmax(axis=1))
+    # EVERY row against the exact result: softmax in fp64 of the fp64 product of
+    # the same bf16 values.  The kernel differs from it by the fp32 summation
+    # of 128 exact products per logit, one v_exp_f32 and one fp32 row sum, so
+    # the bound is the softmax stage's 1e-5, not the bf16 GEMM's 1e-2.
+    worst = 0.0
+    for r0 in range(0, M, 512):
+        logits = (qv[r0:r0 + 512].astype(np.float64) @ kv.T.astype(np.float64)) * float(scale)
+        e = np.exp(logits - logits.max(axis=1, keepdims=True))
+        exact = e / e.sum(axis=1, keepdims=True)
+        worst = max(worst, float(np.max(np.abs(got[r0:r0 + 512] - exact) / exact)))
+    print("qk softmax 4096x4096x128: max relative error against fp64 = %.3g" % worst)
+    assert worst < 1e-5
+
+
+def test_qk_softmax_wide_logit_spread(gpu, oracle):
+    # With scale 2 the logits of a row spread over more than 200, so many
+    # probabilities fall below 2^-126.  The kernel computes exp as v_exp_f32 of
+    # logits held in log2 units, which returns 0 where expf on the CPU returns
+    # a subnormal number: there the two differ by at most the smallest normal
+    # number, everywhere else by the usual relative bound.
+    M, N, D = 64, 2048, 128
+    qb, _ = oracle.to_bf16(oracle.normal((M, D), 15))
+    kb, _ = oracle.to_bf16(oracle.normal((N, D), 16))
+    scale = np.float32(2.0)
+    got = _run_qk(gpu, qb, kb, scale, 2048)
+    want = oracle.qk_softmax(qb, kb, scale)
+    assert np.any((want > 0) & (want < 2.0 ** -126)) and np.any(want > 0.5)
+    assert np.all(np.isfinite(got)) and np.all(got >= 0)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-2 * want.astype(np.float64) + 2.0 ** -126)
+    assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
 
 
 def test_qk_softmax_argument_errors(gpu):
