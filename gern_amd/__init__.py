@@ -20,6 +20,7 @@ NO_XCD_REMAP = 2
 GEMM_OVERWRITE = 4
 GEMM_GENERAL_ONLY = 8
 BLUR_PLAIN_STORES = 16
+QK_ROW_BLOCKS = 32
 
 _libs = None
 

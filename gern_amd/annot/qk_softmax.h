@@ -135,13 +135,118 @@ public:
         return f;
     }
     std::vector<std::string> getHeader() override {
-        return {"gernels/qk_softmax.h"};
+        return {"gernels/qk_softmax.h", "gernels/qk_tiles.h"};
     }
 
 private:
     AbstractDataTypePtr Q, K, logits;
     Variable d{"d", Datatype::Int64, true};
     Variable scale{"scale", Datatype::Float32};
+};
+
+// A 256 x 256 tile of scores spread over the eight wavefronts of a workgroup
+// (gernels/qk_tiles.h).
+//   role OUTPUT : a window of the result matrix in HBM (stored on insert)
+//   role TEMP   : registers only
+class ScoreTileF32 : public TableADT {
+public:
+    enum Role { OUTPUT, TEMP };
+    ScoreTileF32(const std::string &name, Role role)
+        : TableADT(name, role == TEMP ? "auto" : "gernels::MatrixF32") {
+        fields = {x, y, row, col};
+        allocate_call = call("gernels::allocate_score_tile", {}, {row, col});
+        query_call = call("template view_score_tile", {x, y}, {row, col});
+        insert_call = call("store_score_tile", {x, y});
+        query_is_written_back = role == OUTPUT;
+        temporaries_are_freed = false;
+    }
+    bool readMember(const void *object, const std::string &member, int64_t &value) const override {
+        return MatrixF32("", MatrixF32::INPUT).readMember(object, member, value);
+    }
+
+private:
+    Variable x{"x"};
+    Variable y{"y"};
+    Variable row{"row", Datatype::Int64, true};
+    Variable col{"col", Datatype::Int64, true};
+};
+
+// Layout of the object handed to Runner::evaluate for a RowStatsExchange
+// (gernels::RowStatsExchange): device memory, all zeros before its first use.
+struct RowStatsExchangeLayout {
+    void *entries;       // `capacity` entries of 16 bytes: rows (padded to the tile height) x pitch of them are used
+    void *state;         // two 32-bit words
+    int32_t pitch;       // entries per row: at least the number of column blocks
+    int32_t spin_limit;  // polls before a wavefront gives up
+    int64_t capacity;
+};
+
+// Where the workgroups of a row block meet (gernels/qk_tiles.h).  No fields and
+// no subsets; its query opens the launch's session, which the code generator
+// places at the top of the kernel because it depends on no loop.
+class RowStatsExchange : public TableADT {
+public:
+    explicit RowStatsExchange(const std::string &name)
+        : TableADT(name, "gernels::RowStatsExchange") {
+        query_call = call("open");
+        free_call = FunctionSignature{};
+    }
+};
+
+// out = 2^(in - rowmax) with the row statistics of the tile kept beside it.
+class ExpRows : public ExpMatrix {
+public:
+    using ExpMatrix::ExpMatrix;
+    FunctionSignature getFunction() override {
+        FunctionSignature f = ExpMatrix::getFunction();
+        f.name = "gernels::exp_rows";
+        return f;
+    }
+    Annotation getAnnotation() override {
+        Variable x("x"), y("y");
+        Variable l_x("l_x", Datatype::Int64, true), l_y("l_y", Datatype::Int64, true);
+        return Tileable(x = Expr(0), ADTMember(output, "row", false), l_x,
+                        Tileable(y = Expr(0), ADTMember(output, "col", false), l_y,
+                                 Produces::Subset(output, {x, y, l_x, l_y}),
+                                 Consumes::Subset(input, {x, y, l_x, l_y})))
+            .occupies({Grid::Unit::THREAD_X});
+    }
+    std::vector<std::string> getHeader() override {
+        return {"gernels/qk_tiles.h"};
+    }
+};
+
+// out = in scaled per row to the softmax of the WHOLE row; the tiles of a row
+// block exchange their statistics through `exchange`.
+class NormaliseRows : public AbstractFunction {
+public:
+    NormaliseRows(AbstractDataTypePtr input, AbstractDataTypePtr exchange, AbstractDataTypePtr output)
+        : input(input), exchange(exchange), output(output) {
+    }
+    Annotation getAnnotation() override {
+        Variable x("x"), y("y");
+        Variable l_x("l_x", Datatype::Int64, true), l_y("l_y", Datatype::Int64, true);
+        return Tileable(x = Expr(0), ADTMember(output, "row", false), l_x,
+                        Tileable(y = Expr(0), ADTMember(output, "col", false), l_y,
+                                 Produces::Subset(output, {x, y, l_x, l_y}),
+                                 Consumes::Subsets(SubsetObjMany({
+                                     SubsetObj(input, {x, y, l_x, l_y}),
+                                     SubsetObj(exchange, {}),
+                                 }))))
+            .occupies({Grid::Unit::THREAD_X});
+    }
+    FunctionSignature getFunction() override {
+        FunctionSignature f;
+        f.name = "gernels::normalise_rows";
+        f.args = {Parameter(input), Parameter(exchange), Parameter(output)};
+        return f;
+    }
+    std::vector<std::string> getHeader() override {
+        return {"gernels/qk_tiles.h"};
+    }
+
+private:
+    AbstractDataTypePtr input, exchange, output;
 };
 
 // divide_vec for row blocks: a block spans ALL columns of its rows (the row

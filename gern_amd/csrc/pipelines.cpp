@@ -71,6 +71,9 @@ struct gern_pipeline_s {
     // softmax / qk
     int64_t ncol = 0;
     int64_t head_dim = 0;
+    // qk on 256 x 256 tiles: the memory through which the workgroups of a row block exchange row statistics
+    bool qk_tiles = false;
+    void *qk_scratch = nullptr;
     // parameter names
     std::vector<std::string> names;
 };
@@ -504,34 +507,61 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
     p->kind = gern_pipeline_s::QK_SOFTMAX;
     p->head_dim = head_dim;
     p->ncol = max_keys;
+    p->qk_tiles = head_dim % 64 == 0 && !(flags & GERN_PIPELINE_QK_ROW_BLOCKS);
     try {
         auto Q = AbstractDataTypePtr(new const annot::MatrixOperand("Q", annot::MatrixOperand::BF16));
         auto K = AbstractDataTypePtr(new const annot::MatrixOperand("K", annot::MatrixOperand::BF16));
-        auto S = AbstractDataTypePtr(new const annot::RowBlockF32("S", annot::RowBlockF32::OUTPUT));
-        auto logits = AbstractDataTypePtr(new const annot::RowBlockF32("logits", annot::RowBlockF32::TEMP));
-        auto shifted = AbstractDataTypePtr(new const annot::RowBlockF32("shifted", annot::RowBlockF32::TEMP));
-        auto expd = AbstractDataTypePtr(new const annot::RowBlockF32("expd", annot::RowBlockF32::TEMP));
-        auto row_max = AbstractDataTypePtr(new const annot::RowStat("row_max"));
-        auto row_sum = AbstractDataTypePtr(new const annot::RowStat("row_sum"));
         Variable rows("rows"), keys("keys"), d("d"), scale("scale", Datatype::Float32), threads("threads");
-        annot::QKScaled qk{Q, K, logits};
-        annot::MaxRow max_row{logits, row_max};
-        annot::SubtractVec sub{row_max, logits, shifted};
-        annot::ExpMatrix ex{shifted, expd};
-        annot::SumRow sum_row{expd, row_sum};
-        annot::DivideVecWholeRows div{row_sum, expd, S};
-        std::map<std::string, Variable> width{{"ncol", keys.bind(max_keys)}};
-        Composable program = Global(
-            (Tile(S["row"], rows.bind(16)) || Grid::BLOCK_X)(Tile(S["col"], keys.bind(max_keys))(
-                qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), max_row[width](row_max, logits),
-                sub(row_max, logits, shifted), ex(shifted, expd), sum_row[width](row_sum, expd),
-                div(row_sum, expd, S))),
-            // gernels/qk_softmax.h, qk_waves(): more wavefronts share a row
-            // block as it gets wider.
-            {{Grid::BLOCK_DIM_X, threads.bind(64 * qkWaves(max_keys))}});
+        Composable program;
+        if (p->qk_tiles) {
+            // 256 x 256 tiles of S, one per workgroup; column blocks along x so that the
+            // workgroups of a row block, which wait for one another, have consecutive ids.
+            using Tile256 = annot::ScoreTileF32;
+            auto S = AbstractDataTypePtr(new const Tile256("S", Tile256::OUTPUT));
+            auto logits = AbstractDataTypePtr(new const Tile256("logits", Tile256::TEMP));
+            auto expd = AbstractDataTypePtr(new const Tile256("expd", Tile256::TEMP));
+            auto exchange = AbstractDataTypePtr(new const annot::RowStatsExchange("exchange"));
+            annot::QKScaled qk{Q, K, logits};
+            annot::ExpRows ex{logits, expd};
+            annot::NormaliseRows norm{expd, exchange, S};
+            program = Global((Tile(S["row"], rows.bind(256)) || Grid::BLOCK_Y)((Tile(S["col"], keys.bind(256)) || Grid::BLOCK_X)(
+                                 qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), ex(logits, expd), norm(expd, exchange, S))),
+                             {{Grid::BLOCK_DIM_X, threads.bind(512)}});
+        } else {
+            auto S = AbstractDataTypePtr(new const annot::RowBlockF32("S", annot::RowBlockF32::OUTPUT));
+            auto logits = AbstractDataTypePtr(new const annot::RowBlockF32("logits", annot::RowBlockF32::TEMP));
+            auto shifted = AbstractDataTypePtr(new const annot::RowBlockF32("shifted", annot::RowBlockF32::TEMP));
+            auto expd = AbstractDataTypePtr(new const annot::RowBlockF32("expd", annot::RowBlockF32::TEMP));
+            auto row_max = AbstractDataTypePtr(new const annot::RowStat("row_max"));
+            auto row_sum = AbstractDataTypePtr(new const annot::RowStat("row_sum"));
+            annot::QKScaled qk{Q, K, logits};
+            annot::MaxRow max_row{logits, row_max};
+            annot::SubtractVec sub{row_max, logits, shifted};
+            annot::ExpMatrix ex{shifted, expd};
+            annot::SumRow sum_row{expd, row_sum};
+            annot::DivideVecWholeRows div{row_sum, expd, S};
+            std::map<std::string, Variable> width{{"ncol", keys.bind(max_keys)}};
+            program = Global(
+                (Tile(S["row"], rows.bind(16)) || Grid::BLOCK_X)(Tile(S["col"], keys.bind(max_keys))(
+                    qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), max_row[width](row_max, logits),
+                    sub(row_max, logits, shifted), ex(shifted, expd), sum_row[width](row_sum, expd),
+                    div(row_sum, expd, S))),
+                // gernels/qk_softmax.h, qk_waves(): more wavefronts share a row
+                // block as it gets wider.
+                {{Grid::BLOCK_DIM_X, threads.bind(64 * qkWaves(max_keys))}});
+        }
         int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
         if (rc != 0) {
             return rc;
+        }
+        if (p->qk_tiles && p->runner) {
+            // Device memory of the exchange, all zeros (gernels/qk_tiles.h); owned by the pipeline.
+            if (gern_hip_malloc(&p->qk_scratch, GERN_QK_SCRATCH_BYTES) != 0 ||
+                gern_hip_memset(p->qk_scratch, 0, GERN_QK_SCRATCH_BYTES) != 0) {
+                std::string msg(gern_hip_last_error(nullptr, 0) + 1, '\0');
+                gern_hip_last_error(msg.data(), msg.size());
+                return fail("gern_qk_softmax_create: " + msg);
+            }
         }
     } catch (const std::exception &e) {
         return fail(e.what());
@@ -540,30 +570,65 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
     return 0;
 }
 
-int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M, int64_t N,
-                        float scale, void *stream) {
+namespace {
+
+// Polls before a wavefront of the tile kernel gives up on the other tiles of its
+// row block (a poll takes a microsecond or two); GERN_QK_SPIN_LIMIT overrides it.
+int32_t qkSpinLimit() {
+    if (const char *forced = std::getenv("GERN_QK_SPIN_LIMIT")) {
+        return (int32_t)std::atol(forced);
+    }
+    return 1 << 18;
+}
+
+}  // namespace
+
+// One run of either QK program; `scratch` (tile program only) is
+// GERN_QK_SCRATCH_BYTES of device memory that no other run uses at the same time.
+// Internal to this library (shared with csrc/qk_no_alloc.hip).
+__attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M, int64_t N,
+                               float scale, void *scratch, void *stream, const char *who) {
+    const std::string name(who);
     if (p == nullptr || p->kind != gern_pipeline_s::QK_SOFTMAX || Q == nullptr || K == nullptr || S == nullptr) {
-        return fail("gern_qk_softmax_run: bad pipeline or null buffer");
+        return fail(name + ": bad pipeline or null buffer");
     }
     if (!p->runner) {
-        return fail("gern_qk_softmax_run: the pipeline was created compile-only");
+        return fail(name + ": the pipeline was created compile-only");
     }
     if (M < 1 || N < 1 || N > p->ncol) {
-        return fail("gern_qk_softmax_run: N exceeds the max_keys the pipeline was created for");
+        return fail(name + ": N exceeds the max_keys the pipeline was created for");
     }
     if (((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K)) & 15u) != 0 || (reinterpret_cast<uintptr_t>(S) & 3u) != 0) {
-        return fail("gern_qk_softmax_run: Q and K are read in 16-byte pieces and must be 16-byte aligned (S 4-byte aligned)");
+        return fail(name + ": Q and K are read in 16-byte pieces and must be 16-byte aligned (S 4-byte aligned)");
     }
     hip::MatrixF32 q{reinterpret_cast<float *>(const_cast<uint16_t *>(Q)), M, p->head_dim, p->head_dim};
     hip::MatrixF32 k{reinterpret_cast<float *>(const_cast<uint16_t *>(K)), N, p->head_dim, p->head_dim};
     hip::MatrixF32 s{S, M, N, N};
     try {
         p->runner->setStream(stream);
-        p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"scale", &scale}});
+        if (!p->qk_tiles) {
+            p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"scale", &scale}});
+            return 0;
+        }
+        // entries: 16 bytes per (row of the padded row count, column block), sixteen column blocks per row
+        const int64_t padded_rows = (M + 255) / 256 * 256;
+        const int64_t pitch = ((N + 255) / 256 + 15) / 16 * 16;
+        const int64_t capacity = ((int64_t)GERN_QK_SCRATCH_BYTES - 256) / 16;
+        if (scratch == nullptr || padded_rows * pitch > capacity) {
+            return fail(name + ": M x N needs more than GERN_QK_SCRATCH_BYTES of exchange memory (M up to 16384 at 4096 keys)");
+        }
+        annot::RowStatsExchangeLayout exchange{static_cast<char *>(scratch) + 256, scratch, (int32_t)pitch, qkSpinLimit(), capacity};
+        p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"exchange", &exchange}, {"scale", &scale}});
     } catch (const std::exception &e) {
         return fail(e.what());
     }
     return 0;
+}
+
+int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M, int64_t N,
+                        float scale, void *stream) {
+    return gern_detail_qk_softmax_run(p, Q, K, S, M, N, scale, p != nullptr ? p->qk_scratch : nullptr, stream,
+                                      "gern_qk_softmax_run");
 }
 
 const char *gern_pipeline_source(gern_pipeline p) {
@@ -593,6 +658,9 @@ int gern_pipeline_destroy(gern_pipeline p) {
             if (r != nullptr) {
                 r->release();
             }
+        }
+        if (p->qk_scratch != nullptr) {
+            gern_hip_free(p->qk_scratch);
         }
     }
     delete p;

@@ -1,0 +1,471 @@
+// Fused S = softmax_rows(scale * Q K^T) on 256 x 256 tiles of S, one per
+// workgroup, for head dimensions that are multiples of 64.
+//
+// The row-block gernels of gernels/qk_softmax.h give a workgroup sixteen whole
+// rows of S, so every workgroup streams ALL of K out of L2 (256 MiB of L2
+// traffic at 4096 x 4096 x 128: half of that kernel's time).  Here a
+// workgroup owns a 256 x 256 tile, reads 64 KiB of Q and 64 KiB of K once, and
+// the workgroups of a row block combine their row statistics through global
+// memory while the tiles wait in registers:
+//
+//   qk_scaled       MFMA: the tile's logits, kept as raw accumulators plus the
+//                   factor that turns them into log2 units
+//   exp_rows        per row of the tile: maximum m, e = 2^(x - m), sum s of e
+//   normalise_rows  publishes (m, s) per row, waits for the same from the
+//                   other tiles of the row block, and scales e by
+//                   2^(m - M) / S with M, S the statistics of the whole row
+//
+// so a softmax over tiled rows is the five stages of the reference's softmax
+// gernels (apps/common/impl/impl.h:7-188: max, subtract, exp, sum, divide) with
+// the two reductions finished across workgroups, as the reference's
+// grid_reduce_total finishes a sum across blocks with a device-scope atomic
+// (gernels/cccl/wrappers/reduce_wrappers.cuh:42-61).
+//
+// Eight wavefronts; wavefront w owns rows [32 w, 32 w + 32) of the tile and all
+// 256 columns, as 2 x 16 v_mfma_f32_16x16x32_bf16 tiles.  MFMA column j of
+// tile tn = 4 g + t stands for key 64 g + 4 j + t, so a lane holds four
+// consecutive columns of S per group g and stores them with one 16-byte store.
+//
+// The exchange.  An entry is two 64-bit words per (row, column block),
+// (m << 32 | tag) and (s << 32 | tag); the tag is the launch's number, which
+// is kept in device memory next to the entries and advanced by the last
+// workgroup of every launch.  A word says by itself whether it belongs to
+// this launch: nothing is cleared between launches, nothing is passed from the
+// host (a captured launch can be replayed), and no counter sits between the
+// writes and the reads.  When the number wraps around (kRowStatsTagPeriod
+// launches) that last workgroup clears all entries, so a tag left behind by an
+// older launch of another shape is never mistaken for a new one.  Entries are
+// written and read with agent-scope atomic accesses, which go to the memory
+// side past the caches that are private to an XCD; no cache is written back
+// or invalidated.  Each wavefront polls the sixteen entries of its own 32
+// rows on its own.  Workgroup ids run along the columns, so the workgroups of
+// a row block are dispatched together; a workgroup waits only for workgroups
+// of its own row block, and those never wait for a later one.  The wait is
+// bounded all the same: after spin_limit polls a wavefront gives up and stores
+// NaN in its rows.
+//
+// Two launches that use the same exchange must not overlap in time.
+#pragma once
+
+#include "gernels/mm.h"
+#include "gernels/softmax.h"
+
+#ifndef GERN_QK_SLEEP
+#define GERN_QK_SLEEP 2
+#endif
+
+namespace gernels {
+
+typedef float score_f32x4_t __attribute__((ext_vector_type(4)));
+
+// Launch numbers run from 0 to kRowStatsTagPeriod - 1; a tag is the number + 1,
+// and 0 is a word that was never written.
+#ifndef GERN_QK_TAG_PERIOD
+#define GERN_QK_TAG_PERIOD 0xFFFFFFFFu
+#endif
+constexpr unsigned int kRowStatsTagPeriod = GERN_QK_TAG_PERIOD;
+
+// What the launch passes by value (the host fills in a struct of the same
+// layout): `entries` holds `capacity` entries of 16 bytes, at least rows x
+// pitch for the padded row count of the launch, pitch >= the number of column
+// blocks; state[0] is the launch number, state[1] counts the workgroups that
+// are done.  All of it starts as zeros.
+struct RowStatsSession {
+    unsigned long long *entries;
+    unsigned int *state;
+    int pitch;
+    int spin_limit;
+    long long capacity;
+    unsigned int tag;
+};
+
+struct RowStatsExchange {
+    unsigned long long *entries;
+    unsigned int *state;
+    int pitch;
+    int spin_limit;
+    long long capacity;
+
+    // Reads the launch number.  The generated kernel calls this before the
+    // first load of the tile, so the round trip hides behind those.
+    __device__ __forceinline__ RowStatsSession open() const {
+        const unsigned int n = __hip_atomic_load(state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return RowStatsSession{entries, state, pitch, spin_limit, capacity, n % kRowStatsTagPeriod + 1u};
+    }
+};
+
+// A 256 x 256 tile of scores spread over eight wavefronts: acc[tm][4 g + t][i]
+// is row 32 w + 16 tm + 4 (lane / 16) + i, column 64 g + 4 (lane % 16) + t,
+// in units of `unit` (value = acc * unit) until exp_rows, plain afterwards.
+// shift / sum: the statistics of the lane's eight rows over the tile's columns.
+template<int64_t R, int64_t C>
+struct ScoreTile {
+    static_assert(R == 256 && C == 256, "score tiles are 256 x 256");
+    static constexpr int64_t rows = R;
+    static constexpr int64_t cols = C;
+    score_f32x4_t acc[2][16];
+    float shift[2][4];
+    float sum[2][4];
+    float unit;
+    int valid_cols;  // columns of the tile that exist (keys)
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+template<int64_t R, int64_t C>
+__device__ __forceinline__ ScoreTile<R, C> allocate_score_tile() {
+    return ScoreTile<R, C>();
+}
+
+template<int64_t R, int64_t C>
+__device__ __forceinline__ ScoreTile<R, C> MatrixF32::view_score_tile(int64_t, int64_t) const {
+    return ScoreTile<R, C>();
+}
+
+template<int64_t R, int64_t C>
+__device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y, const ScoreTile<R, C> &t) const {
+    const int lane = lane_id();
+    const int w = (int)(threadIdx.x / kWaveSize);
+    const int jl = lane % 16;
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int64_t rr = x + 32 * w + 16 * tm + 4 * (lane / 16) + i;
+            if (rr >= row) {
+                continue;
+            }
+            float *p = data + rr * lda;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int64_t cc = y + 64 * g + 4 * jl;
+                const float4 val = make_float4(t.acc[tm][4 * g + 0][i], t.acc[tm][4 * g + 1][i], t.acc[tm][4 * g + 2][i],
+                                               t.acc[tm][4 * g + 3][i]);
+                if (cc + 3 < col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
+                    store_streaming(p + cc, val);
+                } else {
+                    if (cc + 0 < col) p[cc + 0] = val.x;
+                    if (cc + 1 < col) p[cc + 1] = val.y;
+                    if (cc + 2 < col) p[cc + 2] = val.z;
+                    if (cc + 3 < col) p[cc + 3] = val.w;
+                }
+            }
+        }
+    }
+}
+
+// The raw products Q K^T of the tile; S.unit = scale * log2(e).
+//
+// Both operands are loaded straight into LDS (16 bytes per lane, no register
+// round trip) in stages of 64 along the head dimension, two stages in flight
+// from the start: a stage is 256 rows of Q and 256 keys of K, 128 bytes each,
+// with the 16-byte piece c of LDS row r at position c ^ ((r >> 1) & 7), which
+// spreads the sixteen rows of one fragment read over all banks.  LDS row
+// 64 g + 16 t + j of the K stage holds key 64 g + 4 j + t: the sixteen keys of
+// MFMA tile 4 g + t are then sixteen consecutive LDS rows, like the rows of Q.
+// Rows of Q and keys past the end of the matrices are read from the last
+// valid one (rows past the end are never stored, keys past the end are left
+// out of the statistics by exp_rows).
+template<int64_t R, int64_t C, int64_t D>
+__device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false> &Q, const GlobalView<C, D, uint16_t, false> &K,
+                                          ScoreTile<R, C> &S, float scale) {
+    static_assert(D % 64 == 0 && D >= 64, "score tiles stage the head dimension in steps of 64");
+    constexpr int NK = (int)(D / 64);
+    constexpr int HALF = 256 * 128;  // bytes of one operand's stage
+    __shared__ __attribute__((aligned(16))) unsigned char qk_stage_even[2 * HALF];
+    __shared__ __attribute__((aligned(16))) unsigned char qk_stage_odd[2 * HALF];
+    const int lane = lane_id();
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
+
+    S.unit = scale * 1.4426950408889634f;
+    S.valid_cols = (int)K.rows;
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++) {
+#pragma unroll
+        for (int tn = 0; tn < 16; tn++) {
+            S.acc[tm][tn] = score_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    if (Q.rows <= 0 || K.rows <= 0) {  // workgroup-uniform
+        return;
+    }
+    // Wavefront w issues Q instructions 4w .. 4w+3 and K instructions 4w .. 4w+3
+    // (eight LDS rows each) of every stage: descriptor and stage offset in
+    // scalar registers, one lane offset per instruction.
+    constexpr int kRawBuffer = 0x00020000;
+    const int64_t q_bytes = ((int64_t)(Q.rows - 1) * Q.lda + D) * 2, k_bytes = ((int64_t)(K.rows - 1) * K.lda + D) * 2;
+    const __amdgpu_buffer_rsrc_t desc_q =
+        __builtin_amdgcn_make_buffer_rsrc((void *)Q.data, 0, (int)(q_bytes < 0xFFFFFFFFll ? q_bytes : 0xFFFFFFFFll), kRawBuffer);
+    const __amdgpu_buffer_rsrc_t desc_k =
+        __builtin_amdgcn_make_buffer_rsrc((void *)K.data, 0, (int)(k_bytes < 0xFFFFFFFFll ? k_bytes : 0xFFFFFFFFll), kRawBuffer);
+    int off_q[4], off_k[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = 8 * (w * 4 + j) + lane / 8;  // LDS row
+        const int piece = (lane % 8) ^ ((r >> 1) & 7);
+        const int q_row = r < (int)Q.rows - 1 ? r : (int)Q.rows - 1;
+        off_q[j] = (q_row * (int)Q.lda + piece * 8) * 2;
+        int key = 64 * (r / 64) + 4 * (r % 16) + (r / 16) % 4;
+        key = key < (int)K.rows - 1 ? key : (int)K.rows - 1;
+        off_k[j] = (key * (int)K.lda + piece * 8) * 2;
+    }
+    auto issue = [&](int kt, unsigned char *dst) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_q, (__attribute__((address_space(3))) void *)(dst + (w * 4 + j) * 1024), 16,
+                                                     off_q[j], kt * 128, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_k, (__attribute__((address_space(3))) void *)(dst + HALF + (w * 4 + j) * 1024),
+                                                     16, off_k[j], kt * 128, 0, 0);
+        }
+    };
+    // Fragments: lane l holds row / key l % 16 of an MFMA tile and the eight
+    // values 8 (l / 16) .. + 7 of a 32-deep step.  Every LDS address is one
+    // offset from its stage array (the compiler then orders reads of one stage
+    // against the loads into that stage only).
+    const int swz = ((lane % 16) >> 1) & 7;
+    const int a_off = (32 * w + (lane % 16)) * 128;
+    const int b_off = HALF + (lane % 16) * 128;
+    auto compute = [&](const unsigned char *stage) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int pos = ((4 * s + lane / 16) ^ swz) * 16;
+            const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(stage + (a_off + pos));
+            const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(stage + (a_off + 16 * 128 + pos));
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                const bf16x8_t b = *reinterpret_cast<const bf16x8_t *>(stage + (b_off + tn * 16 * 128 + pos));
+                S.acc[0][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, S.acc[0][tn], 0, 0, 0);
+                S.acc[1][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, S.acc[1][tn], 0, 0, 0);
+            }
+        }
+    };
+    issue(0, qk_stage_even);
+    if (NK > 1) {
+        issue(1, qk_stage_odd);
+    }
+#pragma unroll
+    for (int kt = 0; kt < NK; kt++) {
+        // this wavefront's loads of stage kt have landed (those of stage kt + 1,
+        // eight instructions, may still be in flight), then everybody's
+        if (kt + 1 < NK) {
+            __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+        }
+        __builtin_amdgcn_s_barrier();
+        compute((kt & 1) ? qk_stage_odd : qk_stage_even);
+        if (kt + 2 < NK) {
+            // every wavefront is done reading the stage before it is refilled
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+            __builtin_amdgcn_s_barrier();
+            issue(kt + 2, (kt & 1) ? qk_stage_odd : qk_stage_even);
+        }
+    }
+}
+
+// out = 2^(in - m) per row of the tile, m the row's maximum over the tile's
+// valid columns; out.shift = m, out.sum = the sum of the row's 2^(in - m).
+template<int64_t R, int64_t C>
+__device__ __forceinline__ void exp_rows(const ScoreTile<R, C> &in, ScoreTile<R, C> &out) {
+    const int jl = lane_id() % 16;
+    const float unit = in.unit;
+    const bool partial = in.valid_cols < (int)C;  // workgroup-uniform: the last column block only
+    const bool flip = unit < 0.f;                 // a negative scale turns the largest product into the smallest logit
+    out.unit = 1.0f;
+    out.valid_cols = in.valid_cols;
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float x[16];
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                x[tn] = in.acc[tm][tn][i];
+            }
+            if (flip) {
+#pragma unroll
+                for (int tn = 0; tn < 16; tn++) {
+                    x[tn] = -x[tn];
+                }
+            }
+            if (partial) {
+#pragma unroll
+                for (int tn = 0; tn < 16; tn++) {
+                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
+                    x[tn] = key < in.valid_cols ? x[tn] : -__builtin_huge_valf();
+                }
+            }
+            float m = x[0];
+#pragma unroll
+            for (int tn = 1; tn < 16; tn++) {
+                m = __builtin_fmaxf(m, x[tn]);
+            }
+            m = __builtin_fmaxf(m, dpp_move<0xB1>(m));   // the sixteen lanes of a DPP row share the tile's rows
+            m = __builtin_fmaxf(m, dpp_move<0x4E>(m));
+            m = __builtin_fmaxf(m, dpp_move<0x141>(m));
+            m = __builtin_fmaxf(m, dpp_move<0x140>(m));
+            const float a = flip ? -unit : unit;
+            const float shift = m * a;                   // the row's largest logit, log2 units (a >= 0)
+            float s = 0.f;
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                // a masked column is -inf: 2^-inf = 0 unless a == 0 (0 * inf), which the test below catches
+                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(x[tn], a, -shift));
+                if (partial) {
+                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
+                    e = key < in.valid_cols ? e : 0.f;
+                }
+                out.acc[tm][tn][i] = e;
+                s += e;
+            }
+            s += dpp_move<0xB1>(s);
+            s += dpp_move<0x4E>(s);
+            s += dpp_move<0x141>(s);
+            s += dpp_move<0x140>(s);
+            out.shift[tm][i] = shift;
+            out.sum[tm][i] = s;
+        }
+    }
+}
+
+namespace detail {
+
+// The last workgroup of a launch advances the launch number and clears the
+// count; when the number wraps around it first clears every entry (tag 0: never
+// written).  Called by all threads of the workgroup.
+__device__ __forceinline__ void close_row_stats(const RowStatsSession &ex) {
+    __shared__ unsigned int row_stats_wrap;
+    unsigned int next = ex.tag;  // launch number + 1
+    if (threadIdx.x == 0) {
+        const unsigned int total = gridDim.x * gridDim.y * gridDim.z;
+        const unsigned int before = __hip_atomic_fetch_add(ex.state + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = before + 1u == total;
+        row_stats_wrap = last && next == kRowStatsTagPeriod;
+        if (last && next != kRowStatsTagPeriod) {
+            __hip_atomic_store(ex.state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(ex.state, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __syncthreads();
+    if (row_stats_wrap != 0u) {  // workgroup-uniform; once in kRowStatsTagPeriod launches
+        for (long long i = threadIdx.x; i < 2 * ex.capacity; i += blockDim.x) {
+            __hip_atomic_store(ex.entries + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            __hip_atomic_store(ex.state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(ex.state, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+}  // namespace detail
+
+// out = in * 2^(m - M) / S per row, with (m, s) the tile's own statistics of
+// the row and M, S those of the whole row, combined from the column blocks of
+// the row block through `ex`.  The tile's position comes from the workgroup's
+// place in the grid: column blocks along x, row blocks along y.
+template<int64_t R, int64_t C>
+__device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const RowStatsSession &ex, ScoreTile<R, C> &out) {
+    typedef unsigned long long u64;
+    const int lane = lane_id();
+    const int w = (int)(threadIdx.x / kWaveSize);
+    const int jl = lane % 16;
+    const int bj = (int)blockIdx.x, nbj = (int)gridDim.x;
+    const int64_t row0 = (int64_t)blockIdx.y * R + 32 * w + 4 * (lane / 16);
+    const u64 tag = ex.tag;
+    {
+        // lane j < 8 of each DPP row publishes row slot j (tm = j / 4, i = j % 4)
+        float m = in.shift[0][0], s = in.sum[0][0];
+#pragma unroll
+        for (int q = 1; q < 8; q++) {
+            m = jl == q ? in.shift[q / 4][q % 4] : m;
+            s = jl == q ? in.sum[q / 4][q % 4] : s;
+        }
+        if (jl < 8) {
+            u64 *e = ex.entries + 2 * ((row0 + 16 * (jl / 4) + (jl % 4)) * ex.pitch + bj);
+            __hip_atomic_store(e, ((u64)(unsigned int)as_int(m) << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(e + 1, ((u64)(unsigned int)as_int(s) << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // Lane j collects column block j (j + 16, ...) for its eight rows.
+    float big_m[2][4], big_s[2][4];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        big_m[q / 4][q % 4] = -__builtin_huge_valf();
+        big_s[q / 4][q % 4] = 0.f;
+    }
+    bool failed = false;
+    for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
+        const int b = b0 + jl;
+        u64 got_m[8], got_s[8];
+        int spins = 0;
+        for (;;) {
+            bool mine = true;
+            if (b < nbj) {
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const u64 *e = ex.entries + 2 * ((row0 + 16 * (q / 4) + (q % 4)) * ex.pitch + b);
+                    got_m[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    got_s[q] = __hip_atomic_load(e + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    mine = mine && (got_m[q] & 0xFFFFFFFFull) == tag && (got_s[q] & 0xFFFFFFFFull) == tag;
+                }
+            }
+            if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
+                break;
+            }
+            if (++spins > ex.spin_limit) {  // wave-uniform
+                failed = true;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(GERN_QK_SLEEP);
+        }
+        if (b < nbj) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const float m = as_float((int)(unsigned int)(got_m[q] >> 32)), s = as_float((int)(unsigned int)(got_s[q] >> 32));
+                const float top = __builtin_fmaxf(big_m[q / 4][q % 4], m);
+                big_s[q / 4][q % 4] = big_s[q / 4][q % 4] * __builtin_amdgcn_exp2f(big_m[q / 4][q % 4] - top) +
+                                      s * __builtin_amdgcn_exp2f(m - top);
+                big_m[q / 4][q % 4] = top;
+            }
+        }
+    }
+    out.unit = 1.0f;
+    out.valid_cols = in.valid_cols;
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float m = big_m[tm][i];
+            float top = m;
+            top = __builtin_fmaxf(top, dpp_move<0xB1>(top));
+            top = __builtin_fmaxf(top, dpp_move<0x4E>(top));
+            top = __builtin_fmaxf(top, dpp_move<0x141>(top));
+            top = __builtin_fmaxf(top, dpp_move<0x140>(top));
+            // a lane with no column block holds (-inf, 0) and adds 0 * 2^-inf = 0
+            float s = big_s[tm][i] * __builtin_amdgcn_exp2f(m - top);
+            s += dpp_move<0xB1>(s);
+            s += dpp_move<0x4E>(s);
+            s += dpp_move<0x141>(s);
+            s += dpp_move<0x140>(s);
+            float f = __builtin_amdgcn_exp2f(in.shift[tm][i] - top) * (1.0f / s);
+            f = failed ? __builtin_nanf("") : f;
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                out.acc[tm][tn][i] = in.acc[tm][tn][i] * f;
+            }
+        }
+    }
+    detail::close_row_stats(ex);
+}
+
+}  // namespace gernels

@@ -70,6 +70,9 @@ struct MfmaAccF32;
 // Defined in gernels/qk_softmax.h: sixteen full rows of logits in registers.
 template<int64_t R, int64_t N>
 struct RowBlock;
+// Defined in gernels/qk_tiles.h: a 256 x 256 tile of scores spread over a workgroup.
+template<int64_t R, int64_t C>
+struct ScoreTile;
 // Defined in gernels/softmax.h: R full rows spread over the NW wavefronts of a
 // workgroup.
 template<int64_t R, int64_t C, int NW>
@@ -114,6 +117,11 @@ struct MatrixF32 {
     __device__ __forceinline__ RowBlock<R, N> view_row_block(int64_t x, int64_t y) const;
     template<int64_t R, int64_t N>
     __device__ __forceinline__ void store_row_block(int64_t x, int64_t y, const RowBlock<R, N> &t) const;
+    // The same on 256 x 256 tiles (gernels/qk_tiles.h).
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ ScoreTile<R, C> view_score_tile(int64_t x, int64_t y) const;
+    template<int64_t R, int64_t C>
+    __device__ __forceinline__ void store_score_tile(int64_t x, int64_t y, const ScoreTile<R, C> &t) const;
 
     // Rows spread over the wavefronts of a workgroup (gernels/softmax.h).  The
     // wavefront count is part of the name because the code generator pastes

@@ -585,7 +585,21 @@ private:
             by.push_back(Argument(n->method.data));
             const std::string child = n->child.getName();
             adt_depth[child] = depthOf(by);
-            at_depth[adt_depth[child]].push_back(n);
+            auto &level = at_depth[adt_depth[child]];
+            if (adt_depth[child] == 0 && n->method.call.args.empty() && n->method.call.template_args.empty() &&
+                !n->insert) {
+                // A query that takes nothing (it opens a session on a parameter: a
+                // load whose result is needed much later) goes first, behind the
+                // launch declarations, so that its latency hides behind what follows.
+                auto at = level.begin();
+                while (at != level.end() && ((*at)->kind == NodeKind::GridDecl || (*at)->kind == NodeKind::SmemDecl ||
+                                             (*at)->kind == NodeKind::Opaque || (*at)->kind == NodeKind::Assert)) {
+                    ++at;
+                }
+                level.insert(at, n);
+            } else {
+                level.push_back(n);
+            }
             break;
         }
         case NodeKind::Compute: {

@@ -44,8 +44,17 @@ enum {
     GERN_PIPELINE_GEMM_GENERAL_ONLY = 8,
     /* Blur only: every tile stores exactly its own tile_cols columns, also
      * when tile_cols would allow windows moved to whole 128-byte lines. */
-    GERN_PIPELINE_BLUR_PLAIN_STORES = 16
+    GERN_PIPELINE_BLUR_PLAIN_STORES = 16,
+    /* QK^T softmax only: sixteen whole rows of S per workgroup also for head
+     * dimensions that the 256 x 256 tile kernel takes (multiples of 64). */
+    GERN_PIPELINE_QK_ROW_BLOCKS = 32
 };
+
+/* Device memory through which the workgroups of the QK^T softmax tile kernel
+ * exchange row statistics: 256 bytes of state, then 16 bytes per (row, padded
+ * to a multiple of 256; block of 256 keys, padded to a multiple of sixteen
+ * blocks).  Enough for M = 16384 rows at 4096 keys. */
+#define GERN_QK_SCRATCH_BYTES ((size_t)4 * 1024 * 1024 + 256)
 
 /* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
  * applied left to right ("xy" = horizontal then vertical, "xyx" = the
@@ -100,7 +109,18 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
  * patterns), S is M x N fp32; MFMA tiles feed an in-register row reduction.
  * Q and K 16-byte aligned.
  * head_dim = D (a multiple of 32, at most 256); max_keys bounds N (a multiple
- * of 256, at most 4096: sixteen rows of logits stay in accumulators).
+ * of 256, at most 4096).
+ * D a multiple of 64: one workgroup per 256 x 256 tile of S; the workgroups
+ * of a row block exchange their row maxima and sums through
+ * GERN_QK_SCRATCH_BYTES of device memory that create allocates (the only device
+ * memory this library allocates) and the tiles wait in registers meanwhile.
+ * M x N must fit that memory; runs of ONE pipeline must not overlap in time
+ * (launch them on one stream, or order the streams).  A wavefront that waits
+ * in vain for the rest of its row block (after a second or so: the launch
+ * shares the GPU with something that keeps its partners from starting) stores
+ * NaN in its rows.
+ * Other D (or GERN_PIPELINE_QK_ROW_BLOCKS): sixteen whole rows of S per
+ * workgroup, logits in accumulators, no device memory besides Q, K and S.
  * No counterpart in the reference (it has no bf16 and no matrix-core path);
  * the softmax stages are those of apps/common/annot/functions.h:9-173. */
 int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_pipeline *out);

@@ -149,6 +149,7 @@ def _kernel_notes(tmp_path, make_pipeline):
     ("gemm_bf16", lambda: gern_amd.Gemm("bf16", overwrite=True, flags=gern_amd.COMPILE_ONLY)),
     ("gemm_bf16_accumulate", lambda: gern_amd.Gemm("bf16", flags=gern_amd.COMPILE_ONLY)),
     ("qk_softmax_4096", lambda: gern_amd.QKSoftmax(128, 4096, flags=gern_amd.COMPILE_ONLY)),
+    ("qk_softmax_4096_row_blocks", lambda: gern_amd.QKSoftmax(128, 4096, flags=gern_amd.COMPILE_ONLY | gern_amd.QK_ROW_BLOCKS)),
 ])
 def test_headline_kernels_use_no_scratch_memory(tmp_path, name, make):
     # A kernel that spills registers, or keeps an array on the stack, writes to

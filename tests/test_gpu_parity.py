@@ -468,30 +468,119 @@ def test_gemm_rejects_unsupported_bf16_shapes(gpu):
 
 
 # ------------------------------------------------------- QK^T -> softmax ----
-def _run_qk(gpu, qb, kb, scale, max_keys):
+def _run_qk(gpu, qb, kb, scale, max_keys, flags=0):
     import torch
-    p = gpu.QKSoftmax(qb.shape[1], max_keys)
+    p = gpu.QKSoftmax(qb.shape[1], max_keys, flags=flags)
     S = torch.full((qb.shape[0], kb.shape[0]), float("nan"), dtype=torch.float32, device="cuda")
     p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, scale)
     torch.cuda.synchronize()
     return S.cpu().numpy()
 
 
-# head dimensions 32, 64, 128 and 256 stream K through LDS (256: two tiles in
-# flight instead of four), 96 takes the register path; ragged rows and keys
-@pytest.mark.parametrize("M,N,D,max_keys", [(64, 256, 128, 256), (50, 200, 64, 256), (16, 1024, 128, 1024),
-                                            (37, 1000, 32, 1024), (33, 500, 256, 512), (20, 300, 96, 512),
-                                            (48, 2048, 256, 2048)])
-def test_qk_softmax_matches_oracle(gpu, oracle, M, N, D, max_keys):
+# Head dimensions 64, 128, 192 and 256 take the 256 x 256 tile kernel (row
+# statistics exchanged between workgroups), 32 and 96 the row-block kernel
+# (32: K streamed through LDS, 96: the register path); flag 32
+# (GERN_PIPELINE_QK_ROW_BLOCKS) keeps the row-block kernel for the others too
+# (256: two tiles in flight instead of four).  Ragged rows and keys.
+@pytest.mark.parametrize("M,N,D,max_keys,flags", [(64, 256, 128, 256, 0), (50, 200, 64, 256, 0), (16, 1024, 128, 1024, 0),
+                                                  (37, 1000, 32, 1024, 0), (33, 500, 256, 512, 0), (20, 300, 96, 512, 0),
+                                                  (48, 2048, 256, 2048, 0), (300, 1000, 192, 1024, 0), (513, 257, 64, 512, 0),
+                                                  (700, 4096, 128, 4096, 0),
+                                                  (64, 256, 128, 256, 32), (50, 200, 64, 256, 32), (33, 500, 256, 512, 32),
+                                                  (48, 2048, 256, 2048, 32)])
+def test_qk_softmax_matches_oracle(gpu, oracle, M, N, D, max_keys, flags):
     qb, _ = oracle.to_bf16(oracle.normal((M, D), 5))
     kb, _ = oracle.to_bf16(oracle.normal((N, D), 6))
     scale = np.float32(1.0 / np.sqrt(D))
-    got = _run_qk(gpu, qb, kb, scale, max_keys)
+    got = _run_qk(gpu, qb, kb, scale, max_keys, flags)
     want = oracle.qk_softmax(qb, kb, scale)
     # the bf16-GEMM tolerance governs: inputs are identical bf16 values, the
     # logits differ only by fp32 summation order
     assert np.max(np.abs(got - want) / want) < 1e-2
     assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
+
+
+def test_qk_softmax_tile_kernel_over_changing_shapes_and_scales(gpu, oracle):
+    # One pipeline, one exchange memory: every launch tags its entries with its
+    # own number, so shapes may change from run to run (entries left by a wider
+    # or taller run are never mistaken for this run's), the scale may be
+    # negative (the largest product is then the smallest logit) or zero
+    # (a uniform row), and a graph of launches needs nothing from the host.
+    import torch
+    D = 128
+    p = gpu.QKSoftmax(D, 4096)
+    assert "view_score_tile" in p.source
+    for n, (M, N, scale) in enumerate([(600, 4096, 0.088), (100, 300, 0.088), (600, 4096, -0.05), (257, 1025, 0.0),
+                                       (1024, 2048, 0.088), (16, 256, 0.3), (600, 4096, 0.088)]):
+        qb, _ = oracle.to_bf16(oracle.normal((M, D), 30 + n))
+        kb, _ = oracle.to_bf16(oracle.normal((N, D), 50 + n))
+        S = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        for _ in range(3):  # back-to-back launches of one shape, then the next shape
+            p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, np.float32(scale))
+        torch.cuda.synchronize()
+        got = S.cpu().numpy()
+        want = oracle.qk_softmax(qb, kb, np.float32(scale))
+        assert np.max(np.abs(got - want) / want) < 1e-2, (M, N, scale)
+        assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5), (M, N, scale)
+
+
+def test_qk_softmax_tile_kernel_launch_number_wraps_around(gpu, oracle, monkeypatch):
+    # A tag is the launch number; when the number wraps around, the last
+    # workgroup of that launch clears every entry, so the entries that a tall
+    # launch left behind one period ago are not taken for those of the current
+    # one.  The period is 2^32 - 1 launches; this pipeline is built with 1000.
+    import torch
+    D = 64
+    monkeypatch.setenv("GERN_PIPELINE_EXTRA_OPTIONS", "-DGERN_QK_TAG_PERIOD=1000u")
+    p = gpu.QKSoftmax(D, 512)
+    monkeypatch.delenv("GERN_PIPELINE_EXTRA_OPTIONS")
+    big = (oracle.to_bf16(oracle.normal((600, D), 71))[0], oracle.to_bf16(oracle.normal((512, D), 72))[0])
+    small = (oracle.to_bf16(oracle.normal((8, D), 73))[0], oracle.to_bf16(oracle.normal((256, D), 74))[0])
+    scale = np.float32(0.125)
+
+    def run(qb, kb, times):
+        S = torch.full((qb.shape[0], kb.shape[0]), float("nan"), dtype=torch.float32, device="cuda")
+        dq, dk = _dev(qb.view(np.int16)), _dev(kb.view(np.int16))
+        for _ in range(times):
+            p(dq, dk, S, scale)
+        torch.cuda.synchronize()
+        return S.cpu().numpy()
+
+    want_big = oracle.qk_softmax(big[0], big[1], scale)
+    assert np.max(np.abs(run(*big, 3) - want_big) / want_big) < 1e-2          # launches 0-2: tags 1-3 in 768 x 2 entries
+    want_small = oracle.qk_softmax(small[0], small[1], scale)
+    assert np.max(np.abs(run(*small, 1000) - want_small) / want_small) < 1e-2  # past the wrap: launch number 3 again
+    for times in (1, 1, 1, 995, 3):                                            # launch numbers 3, 4, 5, ..., across the next wrap
+        assert np.max(np.abs(run(*big, times) - want_big) / want_big) < 1e-2
+
+
+def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, monkeypatch):
+    # With no polls allowed, a wavefront that does not find the statistics of
+    # the whole row block at its first look gives up and stores NaN in its
+    # rows: the launch still finishes, every row is either right or NaN, and
+    # the next launch (with the normal limit) is right everywhere.
+    import torch
+    M, N, D = 1024, 4096, 128
+    qb, _ = oracle.to_bf16(oracle.normal((M, D), 5))
+    kb, _ = oracle.to_bf16(oracle.normal((N, D), 6))
+    scale = np.float32(1.0 / np.sqrt(D))
+    want = oracle.qk_softmax(qb, kb, scale)
+    p = gpu.QKSoftmax(D, 4096)
+    dq, dk = _dev(qb.view(np.int16)), _dev(kb.view(np.int16))
+    S = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    monkeypatch.setenv("GERN_QK_SPIN_LIMIT", "0")
+    p(dq, dk, S, scale)
+    torch.cuda.synchronize()
+    got = S.cpu().numpy()
+    bad = np.isnan(got)
+    assert np.all(np.abs(got[~bad] - want[~bad]) / want[~bad] < 1e-2)
+    # NaNs come as whole 256-column pieces of rows (one wavefront's rows of one tile)
+    assert np.array_equal(bad, np.repeat(bad[:, ::256], 256, axis=1))
+    monkeypatch.delenv("GERN_QK_SPIN_LIMIT")
+    p(dq, dk, S, scale)
+    torch.cuda.synchronize()
+    got = S.cpu().numpy()
+    assert np.max(np.abs(got - want) / want) < 1e-2
 
 
 def test_qk_softmax_full_size(gpu, oracle):
