@@ -69,6 +69,7 @@ def _load():
     if hasattr(pipes, "gern_qk_softmax_create"):
         pipes.gern_qk_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
         pipes.gern_qk_softmax_run.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
+        pipes.gern_qk_softmax_run_no_alloc.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
     cpp = C.POINTER(C.c_char_p)
     hip.gern_hip_compile.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(vp)]
     hip.gern_hip_compile_only.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(sz)]
@@ -252,10 +253,12 @@ class QKSoftmax(_Pipeline):
         self.head_dim = head_dim
         _check(pipelines_lib().gern_qk_softmax_create(head_dim, max_keys, flags, C.byref(self.h)))
 
-    def __call__(self, Q, K, S, scale, stream=None):
+    def __call__(self, Q, K, S, scale, stream=None, no_alloc=False):
+        """no_alloc=True: gern_qk_softmax_run_no_alloc (exchange memory from the library's device array)."""
         M, D = Q.shape
         N = K.shape[0]
         assert D == self.head_dim and K.shape[1] == D and tuple(S.shape) == (M, N)
         assert Q.is_contiguous() and K.is_contiguous() and S.is_contiguous()
-        _check(pipelines_lib().gern_qk_softmax_run(self.h, _ptr(Q), _ptr(K), _ptr(S), M, N, float(scale), stream))
+        run = pipelines_lib().gern_qk_softmax_run_no_alloc if no_alloc else pipelines_lib().gern_qk_softmax_run
+        _check(run(self.h, _ptr(Q), _ptr(K), _ptr(S), M, N, float(scale), stream))
         return S

@@ -37,8 +37,13 @@ def build_native():
     srcs = sorted(glob.glob(os.path.join(HERE, "src", "*.cpp")))
     run(["g++"] + CXXFLAGS + ["-shared"] + srcs + ["-L" + HERE, "-lgern_hip", "-ldl", rpath,
                                                   "-o", os.path.join(HERE, "libgern.so")])
-    run(["g++"] + CXXFLAGS + ["-shared", os.path.join(HERE, "csrc", "pipelines.cpp"), "-L" + HERE, "-lgern",
-                               "-lgern_hip", "-ldl", rpath, "-o", os.path.join(HERE, "libgern_pipelines.so")])
+    # The one file of the library with device code of its own (a device array): hipcc, linked in as an object.
+    no_alloc = os.path.join(HERE, "csrc", "qk_no_alloc.o")
+    run([os.path.join(ROCM, "bin", "hipcc")] + HIPFLAGS + ["-fPIC", "-I" + os.path.join(ROOT, "include"), "-c",
+                                                          os.path.join(HERE, "csrc", "qk_no_alloc.hip"), "-o", no_alloc])
+    run(["g++"] + CXXFLAGS + ["-shared", os.path.join(HERE, "csrc", "pipelines.cpp"), no_alloc, "-L" + HERE, "-lgern",
+                               "-lgern_hip", "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-ldl", rpath, "-o",
+                               os.path.join(HERE, "libgern_pipelines.so")])
 
 
 def build_gernel_check():

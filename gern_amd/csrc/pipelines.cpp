@@ -583,6 +583,11 @@ int32_t qkSpinLimit() {
 
 }  // namespace
 
+// Sets the calling thread's error message (for csrc/qk_no_alloc.hip).
+__attribute__((visibility("hidden"))) int gern_detail_fail(const char *message) {
+    return fail(message);
+}
+
 // One run of either QK program; `scratch` (tile program only) is
 // GERN_QK_SCRATCH_BYTES of device memory that no other run uses at the same time.
 // Internal to this library (shared with csrc/qk_no_alloc.hip).

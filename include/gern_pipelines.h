@@ -127,6 +127,19 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
 int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M,
                         int64_t N, float scale, void *stream);
 
+/* gern_qk_softmax_run with the exchange memory taken from a device array of
+ * this library (GERN_QK_SCRATCH_BYTES, one copy per GPU, held from the first
+ * call on that GPU until the process ends) instead of the pipeline's own
+ * allocation: the call allocates nothing on the device, for callers that must
+ * not (a stream under HIP graph capture, a serving loop that forbids it).
+ * Same arguments, same limits (M x N must fit GERN_QK_SCRATCH_BYTES), same
+ * results.  All pipelines of a process share the array of a GPU: calls of this
+ * function that overlap in time on one GPU race (launch them on one stream,
+ * or order the streams); calls of gern_qk_softmax_run do not touch it.
+ * No counterpart in the reference. */
+int gern_qk_softmax_run_no_alloc(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S,
+                                 int64_t M, int64_t N, float scale, void *stream);
+
 /* The generated device source (owned by the pipeline, valid until destroy).
  * A pipeline that holds more than one kernel (the GEMMs) reports the one its
  * last run used; before any run, the faster one. */
