@@ -174,7 +174,7 @@ private:
 // Layout of the object handed to Runner::evaluate for a RowStatsExchange
 // (gernels::RowStatsExchange): device memory, all zeros before its first use.
 struct RowStatsExchangeLayout {
-    void *entries;       // `capacity` entries of 16 bytes: rows (padded to the tile height) x pitch of them are used
+    void *entries;       // `capacity` entries of 8 bytes: rows (padded to the tile height) x pitch of them are used
     void *state;         // two 32-bit words
     int32_t pitch;       // entries per row: at least the number of column blocks
     int32_t spin_limit;  // polls before a wavefront gives up

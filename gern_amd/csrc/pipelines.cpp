@@ -615,10 +615,10 @@ __attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeli
             p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"scale", &scale}});
             return 0;
         }
-        // entries: 16 bytes per (row of the padded row count, column block), sixteen column blocks per row
+        // entries: 8 bytes per (row of the padded row count, column block), sixteen column blocks per row
         const int64_t padded_rows = (M + 255) / 256 * 256;
         const int64_t pitch = ((N + 255) / 256 + 15) / 16 * 16;
-        const int64_t capacity = ((int64_t)GERN_QK_SCRATCH_BYTES - 256) / 16;
+        const int64_t capacity = ((int64_t)GERN_QK_SCRATCH_BYTES - 256) / 8;
         if (scratch == nullptr || padded_rows * pitch > capacity) {
             return fail(name + ": M x N needs more than GERN_QK_SCRATCH_BYTES of exchange memory (M up to 16384 at 4096 keys)");
         }

@@ -26,23 +26,30 @@
 // tile tn = 4 g + t stands for key 64 g + 4 j + t, so a lane holds four
 // consecutive columns of S per group g and stores them with one 16-byte store.
 //
-// The exchange.  An entry is two 64-bit words per (row, column block),
-// (m << 32 | tag) and (s << 32 | tag); the tag is the launch's number, which
-// is kept in device memory next to the entries and advanced by the last
-// workgroup of every launch.  A word says by itself whether it belongs to
-// this launch: nothing is cleared between launches, nothing is passed from the
-// host (a captured launch can be replayed), and no counter sits between the
-// writes and the reads.  When the number wraps around (kRowStatsTagPeriod
-// launches) that last workgroup clears all entries, so a tag left behind by an
-// older launch of another shape is never mistaken for a new one.  Entries are
-// written and read with agent-scope atomic accesses, which go to the memory
-// side past the caches that are private to an XCD; no cache is written back
-// or invalidated.  Each wavefront polls the sixteen entries of its own 32
+// The exchange.  An entry is one 64-bit word per (row, column block): s in the
+// upper half, below it m as a sixteen-bit integer (exp_rows shifts a row by
+// the floor of its largest logit in log2 units: any shift near the maximum
+// serves, and a whole number makes 2^(m - M) an exact power of two), and a
+// sixteen-bit tag.  The tag is the launch's number, which is kept in device
+// memory next to the entries and advanced by the last wavefront of every
+// launch.  An entry says by itself whether it belongs to this launch: nothing
+// is cleared between launches, nothing is passed from the host (a captured
+// launch can be replayed), and no counter sits between the writes and the
+// reads.  When the number wraps around (kRowStatsTagPeriod launches) that last
+// wavefront clears all entries, so a tag left behind by an older launch of
+// another shape is never mistaken for a new one.  Entries are written and read
+// with agent-scope atomic accesses, which go to the memory side past the
+// caches that are private to an XCD; no cache is written back or invalidated.
+// Such reads run at about 3 TB/s over the whole GPU, and every tile reads the
+// entries of its whole row block, so the size of an entry is what the exchange
+// costs: 8 MiB and 2.5 us at 4096 x 4096 (entries of 16 bytes that held m as a
+// float: twice that).  Each wavefront polls the sixteen entries of its own 32
 // rows on its own.  Workgroup ids run along the columns, so the workgroups of
 // a row block are dispatched together; a workgroup waits only for workgroups
 // of its own row block, and those never wait for a later one.  The wait is
 // bounded all the same: after spin_limit polls a wavefront gives up and stores
-// NaN in its rows.
+// NaN in its rows.  Logits beyond +-32767 in log2 units (22 000 in natural
+// units) do not fit an entry; their rows come out as NaN.
 //
 // Two launches that use the same exchange must not overlap in time.
 #pragma once
@@ -61,12 +68,12 @@ typedef float score_f32x4_t __attribute__((ext_vector_type(4)));
 // Launch numbers run from 0 to kRowStatsTagPeriod - 1; a tag is the number + 1,
 // and 0 is a word that was never written.
 #ifndef GERN_QK_TAG_PERIOD
-#define GERN_QK_TAG_PERIOD 0xFFFFFFFFu
+#define GERN_QK_TAG_PERIOD 65535u
 #endif
 constexpr unsigned int kRowStatsTagPeriod = GERN_QK_TAG_PERIOD;
 
 // What the launch passes by value (the host fills in a struct of the same
-// layout): `entries` holds `capacity` entries of 16 bytes, at least rows x
+// layout): `entries` holds `capacity` entries of 8 bytes, at least rows x
 // pitch for the padded row count of the launch, pitch >= the number of column
 // blocks; state[0] is the launch number, state[1] counts the workgroups that
 // are done.  All of it starts as zeros.
@@ -93,6 +100,17 @@ struct RowStatsExchange {
         return RowStatsSession{entries, state, pitch, spin_limit, capacity, n % kRowStatsTagPeriod + 1u};
     }
 };
+
+namespace detail {
+// Wavefronts of the workgroup that are done with the exchange.  qk_scaled clears
+// it ahead of its first barrier and normalise_rows counts in it, so that
+// normalise_rows needs no barrier of its own: the wavefronts of a workgroup
+// finish exp_rows up to a microsecond or two apart (a SIMD serves its older
+// wavefront first), and a wavefront exchanges only with its namesakes in the
+// other tiles of the row block, so the early ones are storing their rows while
+// the late ones still compute.
+__shared__ unsigned int row_stats_waves_done;
+}  // namespace detail
 
 // A 256 x 256 tile of scores spread over eight wavefronts: acc[tm][4 g + t][i]
 // is row 32 w + 16 tm + 4 (lane / 16) + i, column 64 g + 4 (lane % 16) + t,
@@ -187,7 +205,11 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
             S.acc[tm][tn] = score_f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
     }
+    if (threadIdx.x == 0) {
+        detail::row_stats_waves_done = 0u;  // seen by all after the first barrier below
+    }
     if (Q.rows <= 0 || K.rows <= 0) {  // workgroup-uniform
+        __syncthreads();
         return;
     }
     // Wavefront w issues Q instructions 4w .. 4w+3 and K instructions 4w .. 4w+3
@@ -309,7 +331,9 @@ __device__ __forceinline__ void exp_rows(const ScoreTile<R, C> &in, ScoreTile<R,
             m = __builtin_fmaxf(m, dpp_move<0x141>(m));
             m = __builtin_fmaxf(m, dpp_move<0x140>(m));
             const float a = flip ? -unit : unit;
-            const float shift = m * a;                   // the row's largest logit, log2 units (a >= 0)
+            // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
+            // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
+            const float shift = __builtin_fminf(__builtin_fmaxf(__builtin_floorf(m * a), -32768.0f), 32767.0f);
             float s = 0.f;
 #pragma unroll
             for (int tn = 0; tn < 16; tn++) {
@@ -336,31 +360,39 @@ namespace detail {
 
 // The last workgroup of a launch advances the launch number and clears the
 // count; when the number wraps around it first clears every entry (tag 0: never
-// written).  Called by all threads of the workgroup.
-__device__ __forceinline__ void close_row_stats(const RowStatsSession &ex) {
-    __shared__ unsigned int row_stats_wrap;
-    unsigned int next = ex.tag;  // launch number + 1
-    if (threadIdx.x == 0) {
-        const unsigned int total = gridDim.x * gridDim.y * gridDim.z;
-        const unsigned int before = __hip_atomic_fetch_add(ex.state + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last = before + 1u == total;
-        row_stats_wrap = last && next == kRowStatsTagPeriod;
-        if (last && next != kRowStatsTagPeriod) {
-            __hip_atomic_store(ex.state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(ex.state, next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+// written).  Every wavefront calls this once it no longer reads entries;
+// `waves_done` is a zeroed counter in LDS.  Only the last wavefront of a
+// workgroup goes on to the device-wide count (and waits for its answer), so the
+// others start storing their rows at once.
+__device__ __forceinline__ void close_row_stats(const RowStatsSession &ex, unsigned int *waves_done) {
+    const int lane = lane_id();
+    unsigned int seen = 0;
+    if (lane == 0) {
+        seen = __hip_atomic_fetch_add(waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    __syncthreads();
-    if (row_stats_wrap != 0u) {  // workgroup-uniform; once in kRowStatsTagPeriod launches
-        for (long long i = threadIdx.x; i < 2 * ex.capacity; i += blockDim.x) {
+    seen = (unsigned int)__builtin_amdgcn_readfirstlane((int)seen);
+    if (seen + 1u != blockDim.x / kWaveSize) {  // wave-uniform
+        return;
+    }
+    const unsigned int total = gridDim.x * gridDim.y * gridDim.z;
+    const unsigned int next = ex.tag;  // launch number + 1
+    unsigned int before = 0;
+    if (lane == 0) {
+        before = __hip_atomic_fetch_add(ex.state + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    before = (unsigned int)__builtin_amdgcn_readfirstlane((int)before);
+    if (before + 1u != total) {
+        return;
+    }
+    if (next == kRowStatsTagPeriod) {  // once in kRowStatsTagPeriod launches: every other wavefront of the launch is done with the entries
+        for (long long i = lane; i < ex.capacity; i += kWaveSize) {
             __hip_atomic_store(ex.entries + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __builtin_amdgcn_s_waitcnt(0x0070);
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            __hip_atomic_store(ex.state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(ex.state, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+    }
+    if (lane == 0) {
+        __hip_atomic_store(ex.state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(ex.state, next == kRowStatsTagPeriod ? 0u : next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -388,9 +420,9 @@ __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const 
             s = jl == q ? in.sum[q / 4][q % 4] : s;
         }
         if (jl < 8) {
-            u64 *e = ex.entries + 2 * ((row0 + 16 * (jl / 4) + (jl % 4)) * ex.pitch + bj);
-            __hip_atomic_store(e, ((u64)(unsigned int)as_int(m) << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(e + 1, ((u64)(unsigned int)as_int(s) << 32) | tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u64 *e = ex.entries + ((row0 + 16 * (jl / 4) + (jl % 4)) * ex.pitch + bj);
+            const u64 word = ((u64)(unsigned int)as_int(s) << 32) | ((u64)((unsigned int)(int)m & 0xFFFFu) << 16) | tag;
+            __hip_atomic_store(e, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     // Lane j collects column block j (j + 16, ...) for its eight rows.
@@ -403,20 +435,19 @@ __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const 
     bool failed = false;
     for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
         const int b = b0 + jl;
-        u64 got_m[8], got_s[8];
+        u64 got[8];
         int spins = 0;
         for (;;) {
             bool mine = true;
             if (b < nbj) {
 #pragma unroll
                 for (int q = 0; q < 8; q++) {
-                    const u64 *e = ex.entries + 2 * ((row0 + 16 * (q / 4) + (q % 4)) * ex.pitch + b);
-                    got_m[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    got_s[q] = __hip_atomic_load(e + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const u64 *e = ex.entries + ((row0 + 16 * (q / 4) + (q % 4)) * ex.pitch + b);
+                    got[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
 #pragma unroll
                 for (int q = 0; q < 8; q++) {
-                    mine = mine && (got_m[q] & 0xFFFFFFFFull) == tag && (got_s[q] & 0xFFFFFFFFull) == tag;
+                    mine = mine && (got[q] & 0xFFFFull) == tag;
                 }
             }
             if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
@@ -431,7 +462,7 @@ __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const 
         if (b < nbj) {
 #pragma unroll
             for (int q = 0; q < 8; q++) {
-                const float m = as_float((int)(unsigned int)(got_m[q] >> 32)), s = as_float((int)(unsigned int)(got_s[q] >> 32));
+                const float m = (float)(short)(unsigned short)((got[q] >> 16) & 0xFFFFull), s = as_float((int)(unsigned int)(got[q] >> 32));
                 const float top = __builtin_fmaxf(big_m[q / 4][q % 4], m);
                 big_s[q / 4][q % 4] = big_s[q / 4][q % 4] * __builtin_amdgcn_exp2f(big_m[q / 4][q % 4] - top) +
                                       s * __builtin_amdgcn_exp2f(m - top);
@@ -439,6 +470,7 @@ __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const 
             }
         }
     }
+    detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
     out.unit = 1.0f;
     out.valid_cols = in.valid_cols;
 #pragma unroll
@@ -465,7 +497,6 @@ __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const 
             }
         }
     }
-    detail::close_row_stats(ex);
 }
 
 }  // namespace gernels

@@ -231,10 +231,10 @@ def qk_phases(gern_amd, torch):
     K = inputs.to_bf16_bits(inputs.normal((n, d), 6))
     dQ, dK = torch.from_numpy(Q.view(np.int16)).cuda(), torch.from_numpy(K.view(np.int16)).cuda()
     dS = torch.zeros((m, n), device="cuda")
-    scratch = torch.zeros(4 * 1024 * 1024 + 256, dtype=torch.uint8, device="cuda")
+    scratch = torch.zeros(2 * 1024 * 1024 + 256, dtype=torch.uint8, device="cuda")
     stamps = torch.zeros((256, 8, 2), dtype=torch.int64, device="cuda")
     (k,) = _compile(gern_amd, QK_SRC, ["qk_phases"])
-    ex = Exchange(scratch.data_ptr() + 256, scratch.data_ptr(), 16, 1 << 18, (4 * 1024 * 1024) // 16)
+    ex = Exchange(scratch.data_ptr() + 256, scratch.data_ptr(), 16, int(os.environ.get('GERN_QK_SPIN_LIMIT', 1 << 18)), (2 * 1024 * 1024) // 8)
     args = [Mat(dK.data_ptr(), n, d, d), Mat(dQ.data_ptr(), m, d, d), Mat(dS.data_ptr(), m, n, n), ex,
             C.c_float(1.0 / np.sqrt(d)), C.c_void_p(stamps.data_ptr())]
     us = _event_us(gern_amd, torch, lambda: _launch(gern_amd, k, (16, 16, 1), (512, 1, 1), args), 10, 50)

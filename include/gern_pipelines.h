@@ -51,10 +51,10 @@ enum {
 };
 
 /* Device memory through which the workgroups of the QK^T softmax tile kernel
- * exchange row statistics: 256 bytes of state, then 16 bytes per (row, padded
+ * exchange row statistics: 256 bytes of state, then 8 bytes per (row, padded
  * to a multiple of 256; block of 256 keys, padded to a multiple of sixteen
  * blocks).  Enough for M = 16384 rows at 4096 keys. */
-#define GERN_QK_SCRATCH_BYTES ((size_t)4 * 1024 * 1024 + 256)
+#define GERN_QK_SCRATCH_BYTES ((size_t)2 * 1024 * 1024 + 256)
 
 /* Fused separable box-blur chain.  `pattern` is a string over {'x','y'},
  * applied left to right ("xy" = horizontal then vertical, "xyx" = the
@@ -118,7 +118,7 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
  * (launch them on one stream, or order the streams).  A wavefront that waits
  * in vain for the rest of its row block (after a second or so: the launch
  * shares the GPU with something that keeps its partners from starting) stores
- * NaN in its rows.
+ * NaN in its rows, and so does a row whose logits exceed 22 000 in magnitude.
  * Other D (or GERN_PIPELINE_QK_ROW_BLOCKS): sixteen whole rows of S per
  * workgroup, logits in accumulators, no device memory besides Q, K and S.
  * No counterpart in the reference (it has no bf16 and no matrix-core path);
