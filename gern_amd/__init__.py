@@ -70,6 +70,8 @@ def _load():
         pipes.gern_qk_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
         pipes.gern_qk_softmax_run.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
         pipes.gern_qk_softmax_run_no_alloc.argtypes = [vp, vp, vp, vp, i64, i64, C.c_float, vp]
+    pipes.gern_gemm_schedule_create.argtypes = [C.c_int, C.c_int, C.POINTER(vp)]
+    pipes.gern_gemm_schedule_run.argtypes = [vp, vp, vp, vp, vp]
     cpp = C.POINTER(C.c_char_p)
     hip.gern_hip_compile.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(vp)]
     hip.gern_hip_compile_only.argtypes = [C.c_char_p, cpp, C.c_int, cpp, C.c_int, C.c_char_p, C.POINTER(sz)]
@@ -242,6 +244,25 @@ class Gemm(_Pipeline):
         assert tuple(B.shape) == (K, N) and tuple(Cm.shape) == (M, N)
         assert A.is_contiguous() and B.is_contiguous() and Cm.is_contiguous()
         _check(pipelines_lib().gern_gemm_run(self.h, _ptr(A), _ptr(B), _ptr(Cm), M, N, K, stream))
+        return Cm
+
+
+class GemmSchedule(_Pipeline):
+    """C += A @ B on 1024 x 1024 fp32 matrices through a schedule written at the level of Gern's API
+    (the reference's gernels/mm/kernel_3.cu, kernel_6.cu or kernel_10.cu)."""
+
+    SIZE = 1024
+
+    def __init__(self, schedule, flags=0):
+        super().__init__()
+        self.schedule = schedule
+        _check(pipelines_lib().gern_gemm_schedule_create(schedule, flags, C.byref(self.h)))
+
+    def __call__(self, A, B, Cm, stream=None):
+        n = self.SIZE
+        assert tuple(A.shape) == (n, n) and tuple(B.shape) == (n, n) and tuple(Cm.shape) == (n, n)
+        assert A.is_contiguous() and B.is_contiguous() and Cm.is_contiguous()
+        _check(pipelines_lib().gern_gemm_schedule_run(self.h, _ptr(A), _ptr(B), _ptr(Cm), stream))
         return Cm
 
 

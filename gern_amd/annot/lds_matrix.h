@@ -136,10 +136,43 @@ public:
     }
 };
 
+// The same, staged 16 bytes per lane (gernels::GlobalMatrix::stage_into_smem_vec).
 template<int Row, int Col>
-using MatrixGlobalToSharedVec = MatrixGlobalToShared<Row, Col>;
+class MatrixGlobalToSharedVec : public MatrixGlobalToShared<Row, Col> {
+public:
+    using MatrixGlobalToShared<Row, Col>::MatrixGlobalToShared;
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{.name = "template stage_into_smem_vec", .args = {this->x, this->y}, .template_args = {this->row, this->col}};
+    }
+};
+
+// The same, staged by loads that write LDS directly into a dense tile
+// (gernels::GlobalMatrix::stage_into_smem_flat).
 template<int Row, int Col>
-using MatrixGlobalToSharedFlat = MatrixGlobalToShared<Row, Col>;
+class MatrixGlobalToSharedFlat : public MatrixGlobalToShared<Row, Col> {
+public:
+    using MatrixGlobalToShared<Row, Col>::MatrixGlobalToShared;
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{.name = "template stage_into_smem_flat", .args = {this->x, this->y}, .template_args = {this->row, this->col}};
+    }
+};
+
+// Subsets are per-thread float4 register tiles (the reference's gernels
+// annot::MatrixGPU<Row, Col, Stride>, gernels/mm/gern_annot/adt.h:11-60).
+template<int Row, int Col>
+class MatrixGPUVec : public StaticMatrixGPU<Row, Col> {
+public:
+    using StaticMatrixGPU<Row, Col>::StaticMatrixGPU;
+    FunctionSignature getAllocateFunction() const override {
+        return FunctionSignature{.name = "gernels::allocate_static_vec", .template_args = {this->row, this->col}};
+    }
+    FunctionSignature getQueryFunction() const override {
+        return FunctionSignature{.name = "template query", .args = {this->x, this->y}, .template_args = {this->row, this->col}};
+    }
+    FunctionSignature getInsertFunction() const override {
+        return FunctionSignature{.name = "template insert", .args = {this->x, this->y}, .template_args = {this->row, this->col}};
+    }
+};
 
 // C(i.., j..) += A(i.., k..) * B(k.., j..); bind "k_dim" to the reduction length.
 class MatrixMultiplyScalar : public AbstractFunction {
@@ -174,6 +207,18 @@ public:
 protected:
     AbstractDataTypePtr A, B, C;
     Variable k_dim{"k_dim", Datatype::Int64, true};
+};
+
+// The same on float4 register tiles (gernels::matrix_multiply_reg; the
+// reference's annot::MatrixMultiplyReg, gernels/mm/gern_annot/functions.h:54-75).
+class MatrixMultiplyReg : public MatrixMultiplyScalar {
+public:
+    using MatrixMultiplyScalar::MatrixMultiplyScalar;
+    FunctionSignature getFunction() override {
+        FunctionSignature f = MatrixMultiplyScalar::getFunction();
+        f.name = "gernels::matrix_multiply_reg";
+        return f;
+    }
 };
 
 // The allocator's init call for Global(..., smem_size, LdsManager(smem_size)).

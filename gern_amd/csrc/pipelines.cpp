@@ -5,6 +5,7 @@
 #include "gern_pipelines.h"
 
 #include "annot/blur.h"
+#include "annot/lds_matrix.h"
 #include "annot/mm.h"
 #include "annot/qk_softmax.h"
 #include "annot/softmax.h"
@@ -56,7 +57,7 @@ AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
 }  // namespace
 
 struct gern_pipeline_s {
-    enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX } kind;
+    enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX, GEMM_SCHEDULE } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
     std::unique_ptr<Runner> exact;   // GEMM: the direct-to-LDS matrix-core kernel (rows of A in whole 16-byte pieces)
     std::unique_ptr<Runner> tail;    // fp32 GEMM in overwrite mode: C += of the last K % 4 columns, made on first use
@@ -634,6 +635,105 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
                         float scale, void *stream) {
     return gern_detail_qk_softmax_run(p, Q, K, S, M, N, scale, p != nullptr ? p->qk_scratch : nullptr, stream,
                                       "gern_qk_softmax_run");
+}
+
+// User-level GEMM schedules over the LDS-staged matrices (annot/lds_matrix.h), as the reference's
+// gernels/mm/kernel_3.cu, kernel_6.cu and kernel_10.cu compose them, sized for 64-lane wavefronts.
+int gern_gemm_schedule_create(int schedule, int flags, gern_pipeline *out) {
+    if (out == nullptr) {
+        return fail("gern_gemm_schedule_create: null argument");
+    }
+    *out = nullptr;
+    if (schedule != 3 && schedule != 6 && schedule != 10) {
+        return fail("gern_gemm_schedule_create: schedule must be 3, 6 or 10 (the reference's gernels/mm/kernel_<n>.cu)");
+    }
+    constexpr int N = GERN_GEMM_SCHEDULE_SIZE;
+    auto p = std::make_unique<gern_pipeline_s>();
+    p->kind = gern_pipeline_s::GEMM_SCHEDULE;
+    try {
+        using CType = annot::MatrixGlobalToGlobal<N, N>;
+        // a staged copy of C is written back only if the data structure says its queries are copies
+        struct CWrittenBack : CType {
+            using CType::CType;
+            bool insertQuery() const override {
+                return true;
+            }
+        };
+        AbstractDataTypePtr A, B;
+        AbstractDataTypePtr C(schedule == 10 ? static_cast<const AbstractDataType *>(new const CWrittenBack("C", false))
+                                             : static_cast<const AbstractDataType *>(new const CType("C", false)));
+        if (schedule == 3) {
+            A = AbstractDataTypePtr(new const annot::MatrixGlobalToShared<N, N>("A", false));
+            B = AbstractDataTypePtr(new const annot::MatrixGlobalToShared<N, N>("B", false));
+        } else if (schedule == 6) {
+            A = AbstractDataTypePtr(new const annot::MatrixGlobalToSharedVec<N, N>("A", false));
+            B = AbstractDataTypePtr(new const annot::MatrixGlobalToSharedVec<N, N>("B", false));
+        } else {
+            A = AbstractDataTypePtr(new const annot::MatrixGlobalToSharedFlat<N, N>("A", false));
+            B = AbstractDataTypePtr(new const annot::MatrixGlobalToSharedFlat<N, N>("B", false));
+        }
+        annot::MatrixGlobalToShared<N, N> view_of("A_view", false);
+        annot::MatrixQueryRegNoVector<N, N> in_registers("C_reg", false);
+        Variable k_dim("k_dim"), k_tiled("k_tiled"), block_x("block_x"), block_y("block_y"), thread_x("thread_x"), thread_y("thread_y"),
+            thread_k("thread_k"), warp_x("warp_x"), warp_y("warp_y"), lanes_y("lanes_y"), one_val("one_val"), smem_size("smem_size");
+        k_dim = k_dim.bind(N);
+        annot::MatrixMultiplyScalar mm(A, B, C);
+        auto &mm_sp = mm[{{"k_dim", k_dim}}];
+        Composable program;
+        if (schedule == 10) {
+            // kernel_10.cu:108-131: block tile -> wavefront tile -> one output per lane, register copies of C, A and B
+            Composable per_lane = Stage(
+                C, in_registers.getQueryFunction(), in_registers.getInsertFunction(),
+                Stage(A, in_registers.getQueryFunction(),
+                      Stage(B, in_registers.getQueryFunction(),
+                            Reduce(k_dim, thread_k.bind(8))(Stage(A, view_of.getView(), Stage(B, view_of.getView(), mm_sp(A, B, C)))))));
+            Composable lanes = (Tile(C["row"], thread_x.bind(1)) || Grid::Unit::THREAD_X_IN_WRAPS)(
+                (Tile(C["col"], thread_y.bind(1)) || Grid::Unit::THREAD_Y_IN_WRAPS)(per_lane));
+            Composable waves =
+                (Tile(C["row"], warp_x.bind(64)) || Grid::Unit::WARP_Y)((Tile(C["col"], warp_y.bind(16)) || Grid::Unit::WARP_X)(lanes));
+            program = Global((Tile(C["row"], block_x.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(16)) || Grid::Unit::BLOCK_Y)(
+                                 Reduce(k_dim, k_tiled.bind(64))(Stage(A, Stage(B, waves))))),
+                             {{Grid::Dim::BLOCK_DIM_Y, lanes_y.bind(16)}}, smem_size, annot::LdsManager(smem_size));
+        } else {
+            // kernel_3.cu:61-75 / kernel_6.cu:61-74: block tile staged through LDS, 4 x 4 outputs per thread;
+            // 64 x 64 block tiles make workgroups of 256 threads
+            Composable inner = Stage(A, schedule == 3 ? view_of.getView() : view_of.getViewVec(),
+                                     Stage(B, schedule == 3 ? view_of.getView() : view_of.getViewVec(), mm_sp(A, B, C)));
+            if (schedule == 3) {
+                inner = Reduce(k_dim, one_val.bind(16))(inner);
+            }
+            program = Global((Tile(C["row"], block_x.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(64)) || Grid::Unit::BLOCK_Y)(
+                                 Reduce(k_dim, k_tiled.bind(16))(Stage(A, Stage(B, (Tile(C["row"], thread_x.bind(4)) || Grid::Unit::THREAD_Y)(
+                                                                                       (Tile(C["col"], thread_y.bind(4)) || Grid::Unit::THREAD_X)(inner))))))),
+                             {}, smem_size, annot::LdsManager(smem_size));
+        }
+        int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
+        if (rc != 0) {
+            return rc;
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    *out = p.release();
+    return 0;
+}
+
+int gern_gemm_schedule_run(gern_pipeline p, const float *A, const float *B, float *C, void *stream) {
+    if (p == nullptr || p->kind != gern_pipeline_s::GEMM_SCHEDULE || A == nullptr || B == nullptr || C == nullptr) {
+        return fail("gern_gemm_schedule_run: bad pipeline or null buffer");
+    }
+    if (!p->runner) {
+        return fail("gern_gemm_schedule_run: the pipeline was created compile-only");
+    }
+    hip::GlobalMatrixF32 a{const_cast<float *>(A)}, b{const_cast<float *>(B)}, c{C};
+    int64_t smem = 48 * 1024;
+    try {
+        p->runner->setStream(stream);
+        p->runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"smem_size", &smem}});
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    return 0;
 }
 
 const char *gern_pipeline_source(gern_pipeline p) {

@@ -615,6 +615,19 @@ private:
             }
             const int mine = mapped ? 0 : depth;
             var_depth[n->intervalVariable().getName()] = mine;
+            if (mapped && depth > 0) {
+                // A grid-mapped range inside an unmapped loop: its index does not depend
+                // on the loop, and neither may some of its statements.  Those stay where
+                // they are, in the scope around the loop (a copy made there is written
+                // back when THAT scope ends, after the loop); the range itself only
+                // defines its index, ahead of them.
+                const size_t at = at_depth[0].size();
+                visit(n->body);
+                Node range = *n;
+                range.body = block({});
+                at_depth[0].insert(at_depth[0].begin() + (std::ptrdiff_t)at, make(std::move(range)));
+                break;
+            }
             visit(n->body);
             std::vector<NodePtr> body = at_depth[mine];
             at_depth.erase(mine);

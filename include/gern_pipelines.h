@@ -127,6 +127,20 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
 int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M,
                         int64_t N, float scale, void *stream);
 
+/* User-level GEMM schedules, C += A * B on square fp32 matrices of
+ * GERN_GEMM_SCHEDULE_SIZE rows (row-major, dense): the compositions of the
+ * reference's gernels/mm/kernel_3.cu:61-75 (block tiles staged through LDS one
+ * float per lane, 4 x 4 outputs per thread), kernel_6.cu:61-74 (staged 16
+ * bytes per lane) and kernel_10.cu:108-131 (block -> wavefront -> lane tiling,
+ * operands staged by loads that write LDS directly, register copies per
+ * lane), with tile sizes for 64-lane wavefronts, over the scalar
+ * matrix_multiply gernel.  They exist to run and time schedules written at
+ * the level of Gern's API (gernels/mm/bench.cu:72-89 times such a kernel);
+ * the tuned GEMM is gern_gemm_create.  schedule: 3, 6 or 10. */
+#define GERN_GEMM_SCHEDULE_SIZE 1024
+int gern_gemm_schedule_create(int schedule, int flags, gern_pipeline *out);
+int gern_gemm_schedule_run(gern_pipeline p, const float *A, const float *B, float *C, void *stream);
+
 /* gern_qk_softmax_run with the exchange memory taken from a device array of
  * this library (GERN_QK_SCRATCH_BYTES, one copy per GPU, held from the first
  * call on that GPU until the process ends) instead of the pipeline's own

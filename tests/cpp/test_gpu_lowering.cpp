@@ -24,6 +24,8 @@
 #include "annot/reduce.h"
 
 #include <cstdlib>
+#include <iostream>
+#include <map>
 
 using namespace gern;
 
@@ -54,6 +56,11 @@ static bool build(Runner &run, Composable program) {
         const char *names[1] = {name.c_str()};
         const char *opts[2] = {i1.c_str(), i2.c_str()};
         size_t size = 0;
+        if (std::getenv("GERN_TEST_PRINT_SOURCE") != nullptr) {
+            const auto plan = cg.getLaunchPlan();
+            std::cerr << last_source << "\n// launch: " << name << "  grid (" << plan.grid[0] << ", " << plan.grid[1] << ", " << plan.grid[2]
+                      << ")  block (" << plan.block[0] << ", " << plan.block[1] << ", " << plan.block[2] << ")\n";
+        }
         if (gern_hip_compile_only(last_source.c_str(), names, 1, opts, 2, "gfx950", &size) != 0) {
             impl::hipCheck(1);
         }
@@ -230,6 +237,31 @@ CASE("array.tile_mapped_to_wavefronts") {
     int64_t step_val = 2, blk_val = 6;  // 2 blocks x 3 wavefronts
     REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}, {blk.getName(), &blk_val}}));
     expect_offset(a, b, 1, 12);
+    a.destroy();
+    b.destroy();
+}
+
+CASE("array.tile_mapped_to_lanes_inside_wavefronts") {
+    // WARP_X over THREAD_X_IN_WRAPS: the outer tile picks the wavefront
+    // (threadIdx.x / 64), the inner one the lane inside it (threadIdx.x % 64),
+    // and the block has 64 threads per wavefront however few lanes work.
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    annot::Add1GPU add_1;
+    Variable per_wave("per_wave"), step("step");
+    Composable program = Global(
+        (Tile(out["size"], per_wave) || Grid::Unit::WARP_X)((Tile(out["size"], step) || Grid::Unit::THREAD_X_IN_WRAPS)(add_1(in, out))));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("(threadIdx.x / 64)") != std::string::npos);
+    REQUIRE(last_source.find("(threadIdx.x % 64)") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    impl::ArrayGPU a(96), b(96);
+    a.ascending();
+    int64_t per_wave_val = 32, step_val = 2;  // 3 wavefronts x 16 working lanes x 2 elements
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {per_wave.getName(), &per_wave_val}, {step.getName(), &step_val}}));
+    expect_offset(a, b, 1, 96);
     a.destroy();
     b.destroy();
 }
@@ -459,6 +491,166 @@ CASE("schedule.gemm_staged_through_lds") {  // gernels/mm/kernel_3.cu:13-118 of 
     a.destroy();
     b.destroy();
     c.destroy();
+}
+
+// Fills A with the reference's ascending() pattern (i % 10) and B with another small-integer
+// pattern, runs C += A B through `run` and compares with the host product (exact in any order).
+template<int64_t m, int64_t n, int64_t k>
+static void check_schedule_product(Runner &run, const std::map<std::string, void *> &extra = {}) {
+    impl::MatrixGPU a(m, k, k), b(k, n, n), c(m, n, n);
+    std::vector<float> ha(m * k), hb(k * n);
+    for (int64_t e = 0; e < m * k; e++) {
+        ha[e] = (float)(e % 10);
+    }
+    for (int64_t e = 0; e < k * n; e++) {
+        hb[e] = (float)((e * 7) % 10);
+    }
+    impl::hipCheck(gern_hip_memcpy_h2d(a.data, ha.data(), sizeof(float) * ha.size()));
+    impl::hipCheck(gern_hip_memcpy_h2d(b.data, hb.data(), sizeof(float) * hb.size()));
+    hip::GlobalMatrixF32 pa{a.data}, pb{b.data}, pc{c.data};
+    std::map<std::string, void *> args{{"A", &pa}, {"B", &pb}, {"C", &pc}};
+    args.insert(extra.begin(), extra.end());
+    run.evaluate(args);
+    std::vector<float> got = c.get();
+    for (int64_t i = 0; i < m; i++) {
+        for (int64_t j = 0; j < n; j++) {
+            float want = 0.0f;
+            for (int64_t kk = 0; kk < k; kk++) {
+                want += ha[i * k + kk] * hb[kk * n + j];
+            }
+            REQUIRE_EQ(got[i * n + j], want);
+        }
+    }
+    a.destroy();
+    b.destroy();
+    c.destroy();
+}
+
+CASE("schedule.gemm_staged_16_bytes_per_lane") {  // gernels/mm/kernel_6.cu:13-112 of the reference
+    constexpr int64_t m = 128, n = 128, k = 128;
+    using AType = annot::MatrixGlobalToSharedVec<m, k>;
+    using BType = annot::MatrixGlobalToSharedVec<k, n>;
+    using CType = annot::MatrixGlobalToGlobal<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    AType view_of("A_vec", false);
+    Variable k_dim("k_dim"), k_tiled("k_tiled"), block_x("block_x"), block_y("block_y"), thread_x("thread_x"),
+        thread_y("thread_y"), smem_size("smem_size");
+    block_x = block_x.bind(8);
+    block_y = block_y.bind(8);
+    thread_x = thread_x.bind(4);
+    thread_y = thread_y.bind(4);
+    k_dim = k_dim.bind(k);
+    k_tiled = k_tiled.bind(4);
+    annot::MatrixMultiplyScalar mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    Composable program = Global(
+        (Tile(C["row"], block_x) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y) || Grid::Unit::BLOCK_Y)(Reduce(k_dim, k_tiled)(
+            Stage(A, Stage(B, (Tile(C["row"], thread_x) || Grid::Unit::THREAD_Y)((Tile(C["col"], thread_y) || Grid::Unit::THREAD_X)(
+                                  Stage(A, view_of.getViewVec(), Stage(B, view_of.getViewVec(), mm_sp(A, B, C)))))))))),
+        {}, smem_size, LdsManager(smem_size));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("stage_into_smem_vec") != std::string::npos);
+    REQUIRE(last_source.find("get_view_vec") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    int64_t smem = 32 * 32 * 8 * 2 + 1000;  // the reference's figure
+    check_schedule_product<m, n, k>(run, {{smem_size.getName(), &smem}});
+}
+
+CASE("schedule.gemm_blocks_wavefronts_lanes") {  // gernels/mm/kernel_10.cu:13-172 of the reference
+    // Block tile -> "warp" tile (WARP_Y x WARP_X) -> one output per lane
+    // (THREAD_X_IN_WRAPS x THREAD_Y_IN_WRAPS), A and B staged into LDS by loads that
+    // write it directly, a register copy of C, A and B per lane, and an inner
+    // reduction over windows of those copies.  The reference's constants are for
+    // 32-lane warps (a 32 x 32 patch of threads per "warp"); here a wavefront unit
+    // is 64 wide, and 64 x 16 lanes make the 1024 threads of the workgroup.
+    constexpr int64_t m = 128, n = 128, k = 128;
+    using AType = annot::MatrixGlobalToSharedFlat<m, k>;
+    using BType = annot::MatrixGlobalToSharedFlat<k, n>;
+    // The lane's register copy of C must be written back.  A staged copy is written back only if
+    // the data structure says its queries are copies (insertQuery(), src/codegen/finalizer.cpp:73-76
+    // of the reference; its own MatrixGlobalToGlobal says "just a view", so kernel_10.cu as written
+    // drops the copy, while the kernel generated from it earlier, gernels/mm/bench.cu:41, inserts it).
+    struct CType : annot::MatrixGlobalToGlobal<m, n> {
+        using annot::MatrixGlobalToGlobal<m, n>::MatrixGlobalToGlobal;
+        bool insertQuery() const override {
+            return true;
+        }
+    };
+    using RegType = annot::MatrixQueryRegNoVector<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    AType view_of("A_vec", false);
+    RegType in_registers("C_reg", false);
+    Variable k_dim("k_dim"), k_tiled("k_tiled"), block_x("block_x"), block_y("block_y"), warp_x("warp_x"), warp_y("warp_y"),
+        thread_x("thread_x"), thread_y("thread_y"), thread_k("thread_k"), smem_size("smem_size"), lanes_y("lanes_y");
+    constexpr int64_t BM = 64, BN = 16, BK = 64, WM = 64, WN = 16, TM = 1, TN = 1, TK = 8;
+    block_x = block_x.bind(BM);
+    block_y = block_y.bind(BN);
+    warp_x = warp_x.bind(WM);
+    warp_y = warp_y.bind(WN);
+    thread_x = thread_x.bind(TM);
+    thread_y = thread_y.bind(TN);
+    thread_k = thread_k.bind(TK);
+    k_dim = k_dim.bind(k);
+    k_tiled = k_tiled.bind(BK);
+    annot::MatrixMultiplyScalar mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    // innermost first
+    Composable per_lane = Stage(
+        C, in_registers.getQueryFunction(), in_registers.getInsertFunction(),
+        Stage(A, in_registers.getQueryFunction(),
+              Stage(B, in_registers.getQueryFunction(),
+                    Reduce(k_dim, thread_k)(Stage(A, view_of.getView(), Stage(B, view_of.getView(), mm_sp(A, B, C)))))));
+    Composable lanes = (Tile(C["row"], thread_x) || Grid::Unit::THREAD_X_IN_WRAPS)(
+        (Tile(C["col"], thread_y) || Grid::Unit::THREAD_Y_IN_WRAPS)(per_lane));
+    Composable wavefronts = (Tile(C["row"], warp_x) || Grid::Unit::WARP_Y)((Tile(C["col"], warp_y) || Grid::Unit::WARP_X)(lanes));
+    Composable program = Global((Tile(C["row"], block_x) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y) || Grid::Unit::BLOCK_Y)(
+                                    Reduce(k_dim, k_tiled)(Stage(A, Stage(B, wavefronts))))),
+                                // a wavefront unit in y would claim 64 threads (64 x 64 in all); 16 lanes in y are what WN needs
+                                {{Grid::Dim::BLOCK_DIM_Y, lanes_y.bind(WN / TN)}}, smem_size, LdsManager(smem_size));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("stage_into_smem_flat") != std::string::npos);
+    REQUIRE(last_source.find("(threadIdx.y / 64)") != std::string::npos);
+    REQUIRE(last_source.find("(threadIdx.x % 64)") != std::string::npos);
+    REQUIRE(last_source.find("(threadIdx.y % 64)") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    int64_t smem = 48 * 1024;
+    check_schedule_product<m, n, k>(run, {{smem_size.getName(), &smem}});
+}
+
+CASE("schedule.gemm_float4_register_tiles") {  // gernels/mm/mm_registers.cu:13-88 of the reference
+    constexpr int64_t m = 8, n = 8, k = 8;
+    using AType = annot::MatrixGPUVec<m, k>;
+    using BType = annot::MatrixGPUVec<k, n>;
+    using CType = annot::MatrixGPUVec<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    Variable k_dim("k_dim"), c_row("c_row"), c_col("c_col"), k_tile("k_tile");
+    c_row = c_row.bind(4);
+    c_col = c_col.bind(8);
+    k_tile = k_tile.bind(4);
+    k_dim = k_dim.bind(k);
+    annot::MatrixMultiplyReg mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    Composable program = Global((Tile(C["row"], c_row) || Grid::Unit::THREAD_X)(
+        (Tile(C["col"], c_col) || Grid::Unit::THREAD_Y)(Reduce(k_dim, k_tile)(mm_sp(A, B, C)))));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("matrix_multiply_reg") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    check_schedule_product<m, n, k>(run);
 }
 
 // ---- FunctionPtr on the device -----------------------------------------------------------------

@@ -390,6 +390,34 @@ def test_gemm_f32_other_shapes_keep_the_general_kernel(gpu, oracle, M, N, K):
     assert np.array_equal(dC.cpu().numpy(), ai @ bi)
 
 
+# Schedules written at the level of Gern's API (the reference's gernels/mm/kernel_3.cu:61-75,
+# kernel_6.cu:61-74 and kernel_10.cu:108-131) over the scalar matrix_multiply gernel: every
+# output is one fp32 sum in ascending k, so the oracle's loop order gives the same bits.
+@pytest.mark.parametrize("schedule", [3, 6, 10])
+def test_gemm_user_schedules_match_oracle(gpu, oracle, schedule):
+    import torch
+    n = gpu.GemmSchedule.SIZE
+    g = gpu.GemmSchedule(schedule)
+    ai = np.random.RandomState(61).randint(-3, 4, size=(n, n)).astype(np.float32)
+    bi = np.random.RandomState(62).randint(-3, 4, size=(n, n)).astype(np.float32)
+    c0 = np.random.RandomState(63).randint(-5, 6, size=(n, n)).astype(np.float32)
+    dC = _dev(c0)
+    g(_dev(ai), _dev(bi), dC)
+    torch.cuda.synchronize()
+    assert np.array_equal(dC.cpu().numpy().astype(np.float64), ai.astype(np.float64) @ bi.astype(np.float64) + c0)
+    A = oracle.uniform((n, n), 64, -1.0, 1.0)
+    B = oracle.uniform((n, n), 65, -1.0, 1.0)
+    dC = torch.zeros((n, n), dtype=torch.float32, device="cuda")
+    g(_dev(A), _dev(B), dC)
+    torch.cuda.synchronize()
+    got = dC.cpu().numpy()
+    for rows in ((0, 8), (60, 68), (n - 4, n)):
+        want = oracle.gemm_f32(A, B, rows=rows)[rows[0]:rows[1]]
+        assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(n)
+    want64 = A.astype(np.float64) @ B.astype(np.float64)
+    assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(n)
+
+
 @pytest.mark.parametrize("variant", ["f32", "bf16"])
 def test_gemm_accumulates_into_c(gpu, oracle, variant):
     A = oracle.uniform((192, 128), 3, -1.0, 1.0)
