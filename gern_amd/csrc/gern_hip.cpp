@@ -588,6 +588,28 @@ int gern_hip_module_unload(gern_hip_module module) {
     return GERN_HIP_OK;
 }
 
+int gern_hip_module_global(gern_hip_module module, const char *name, void **ptr, size_t *bytes) {
+    if (module == nullptr || name == nullptr || ptr == nullptr) {
+        return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_module_global: null argument");
+    }
+    *ptr = nullptr;
+    hipDeviceptr_t at = nullptr;
+    size_t size = 0;
+    hipError_t e = hipModuleGetGlobal(&at, &size, module->module, name);
+    if (e == hipErrorNotFound) {
+        (void)hipGetLastError();
+        return GERN_HIP_OK;
+    }
+    if (e != hipSuccess) {
+        return hip_fail(e, (std::string("hipModuleGetGlobal(") + name + ")").c_str());
+    }
+    *ptr = at;
+    if (bytes != nullptr) {
+        *bytes = size;
+    }
+    return GERN_HIP_OK;
+}
+
 int gern_hip_malloc(void **ptr, size_t bytes) {
     if (ptr == nullptr) {
         return fail(GERN_HIP_ERR_ARGUMENT, "gern_hip_malloc: null output pointer");

@@ -60,7 +60,7 @@ struct gern_pipeline_s {
     enum Kind { BLUR, SOFTMAX, GEMM_F32, GEMM_BF16, QK_SOFTMAX, GEMM_SCHEDULE } kind;
     std::unique_ptr<Runner> runner;  // null in compile-only mode
     std::unique_ptr<Runner> exact;   // GEMM: the direct-to-LDS matrix-core kernel (rows of A in whole 16-byte pieces)
-    std::unique_ptr<Runner> tail;    // fp32 GEMM in overwrite mode: C += of the last K % 4 columns, made on first use
+    std::unique_ptr<Runner> tail;    // fp32 GEMM in overwrite mode: C += of the last K % 4 columns
     bool accumulate = true;          // GEMM: C += A * B (false: C = A * B)
     int create_flags = 0;
     std::string source;
@@ -405,6 +405,15 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
             p->exact_kernel_name = fast.kernel_name.empty() && p->exact ? p->exact->getKernelName() : fast.kernel_name;
             // The shape the pipeline is built for is the exact one.
             p->last_run_exact = true;
+            if (rc == 0 && !bf16 && !accumulate) {
+                // An fp32 product whose K is not a multiple of 4 is split in two launches (gern_gemm_run);
+                // the second one ADDS the last columns even when the pipeline overwrites C.  Built here so
+                // that a run never compiles.
+                gern_pipeline_s rest;
+                rc = finish(&rest, gemmProgram(element, false, annot::MatrixAccumulator::FMA, true, 128, 128, 256, 2 * 2 * 16 * 132 * 4),
+                            flags);
+                p->tail = std::move(rest.runner);
+            }
         }
         if (rc != 0) {
             return rc;
@@ -469,17 +478,10 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
         if (k_main < K) {
             Runner *rest = p->runner.get();  // accumulates unless the pipeline overwrites C
             if (!p->accumulate) {
-                if (!p->tail) {
-                    gern_pipeline_s made;
-                    if (finish(&made,
-                               gemmProgram(annot::MatrixOperand::F32, false, annot::MatrixAccumulator::FMA, true, 128, 128, 256,
-                                           2 * 2 * 16 * 132 * 4),
-                               p->create_flags | GERN_PIPELINE_NO_XCD_REMAP) != 0) {
-                        return 1;
-                    }
-                    p->tail = std::move(made.runner);
+                rest = p->tail.get();  // made by gern_gemm_create
+                if (rest == nullptr) {
+                    return fail("gern_gemm_run: the pipeline has no kernel for the last K % 4 columns");
                 }
-                rest = p->tail.get();
             }
             hip::MatrixF32 a2{a.data + k_main, M, K - k_main, K};
             hip::MatrixF32 b2{b.data + k_main * N, K - k_main, N, N};

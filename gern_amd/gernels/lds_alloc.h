@@ -22,6 +22,15 @@ extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 
 constexpr int kLdsMaxBlocks = 14;
 
+}  // namespace gernels
+
+// Requests the allocator could not meet since the code was loaded, over all
+// launches and workgroups.  A word in device memory with an unmangled name, so
+// that the host can find it in the loaded code (Runner::ldsOverflows()).
+extern "C" __device__ unsigned int gern_lds_overflows = 0;
+
+namespace gernels {
+
 // Table at the start of dynamic LDS (128 bytes).  Blocks are kept sorted by
 // offset and cover [first, capacity) without gaps; a block is free or in use.
 struct LdsTable {
@@ -57,7 +66,7 @@ __device__ __forceinline__ void lds_init(int64_t bytes) {
 // overflow flag is set and the START of the heap is returned, so that the
 // caller's accesses stay inside LDS (results are then wrong, as with the
 // reference's allocator once it wraps, but nothing faults).  lds_overflowed()
-// tells.
+// tells the kernel, the count in gern_lds_overflows tells the host.
 __device__ __forceinline__ void *lds_alloc(int64_t bytes) {
     LdsTable *t = reinterpret_cast<LdsTable *>(gern_lds);
     __syncthreads();  // earlier readers of `answer` are done
@@ -88,6 +97,7 @@ __device__ __forceinline__ void *lds_alloc(int64_t bytes) {
         if (got == 0) {
             t->overflow = 1;
             got = (uint32_t)sizeof(LdsTable);
+            atomicAdd(&gern_lds_overflows, 1u);
         }
         t->answer = got;
     }

@@ -40,10 +40,12 @@ extern __shared__ __attribute__((aligned(16))) unsigned char gern_lds[];
 // A window onto a row-major matrix in HBM: at most R x C, of which
 // rows x cols lie inside the matrix.  EXACT is a promise about the matrix the
 // window was cut from, made by the program that declares the operand: the
-// matrix is one dense allocation that ends with its last element, the rows of
-// A start on 16-byte boundaries and hold a whole number of 16-byte pieces (its
-// reduction extent is a multiple of 8 for bf16, of 4 for fp32), the rows of B
-// start on 4-byte boundaries, and row pitches stay below kMfmaMaxLd elements.
+// matrix is one dense allocation that ends with its last element, A starts on
+// a 16-byte boundary and the part of each of its rows that is multiplied is a
+// whole number of 16-byte pieces (the reduction extent is a multiple of 8 for
+// bf16, of 4 for fp32; the rows themselves need only 4-byte alignment, their
+// pitch may be longer than the reduction extent), B starts on a 4-byte
+// boundary, and row pitches stay below kMfmaMaxLd elements.
 // Windows on the bottom and right edges may be partial, and so may the last
 // stage of the reduction: rows and cols say how much of them exists.
 template<int64_t R, int64_t C, typename T, bool EXACT>

@@ -78,6 +78,11 @@ public:
     // that creates Runners over and over calls release() when it is done with
     // one.  The Runner cannot evaluate afterwards.
     void release();
+    // Device launches whose kernel uses the LDS allocator (gernels/lds_alloc.h):
+    // waits for the device, then returns how many requests the allocator could
+    // not meet since the code was loaded (results of such launches are wrong;
+    // give the launch more dynamic LDS).  0 for every other kernel.
+    int64_t ldsOverflows();
 
 private:
     FunctionSignature signature;

@@ -44,6 +44,25 @@ Runner::Runner(Composable c, std::optional<std::vector<Parameter>> ordered_param
     : c(c), ordered_parameters(ordered_parameters) {
 }
 
+int64_t Runner::ldsOverflows() {
+    if (module == nullptr) {
+        return 0;
+    }
+    void *at = nullptr;
+    size_t bytes = 0;
+    uint32_t count = 0;
+    if (gern_hip_module_global(static_cast<gern_hip_module>(module), "gern_lds_overflows", &at, &bytes) != GERN_HIP_OK) {
+        throw error::UserError("Cannot look up the LDS overflow count: " + lastHipError());
+    }
+    if (at == nullptr) {
+        return 0;
+    }
+    if (bytes != sizeof(count) || gern_hip_sync() != GERN_HIP_OK || gern_hip_memcpy_d2h(&count, at, sizeof(count)) != GERN_HIP_OK) {
+        throw error::UserError("Cannot read the LDS overflow count: " + lastHipError());
+    }
+    return count;
+}
+
 Runner::~Runner() {
     // The module stays loaded for the life of the process, like the
     // reference's dlopen handle: kernels may still be in flight.
@@ -183,8 +202,15 @@ void Runner::evaluate(std::map<std::string, void *> args) {
     };
 
     for (const auto &assumption : plan->host_asserts) {
+        // The kernel was compiled to rely on every one of these, so one that cannot be checked
+        // here refuses the launch just as one that fails.
         bool holds = true;
-        if (codegen::evaluate(assumption, env, holds) && !holds) {
+        if (!codegen::evaluate(assumption, env, holds)) {
+            throw error::UserError("Cannot check the assumption " + assumption.str() +
+                                   " on the host: a data structure whose members appear in an assumption of a "
+                                   "device kernel must implement AbstractDataType::readMember");
+        }
+        if (!holds) {
             throw error::UserError("Assumption violated at launch: " + assumption.str());
         }
     }

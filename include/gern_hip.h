@@ -97,6 +97,12 @@ int gern_hip_check(void);
 
 int gern_hip_module_unload(gern_hip_module module);
 
+/* Address and size of a __device__ variable of the loaded code, by its
+ * (unmangled) name.  *ptr is NULL, and the call succeeds, when the code has no
+ * such variable.  No counterpart in the reference, whose generated code holds
+ * no device variables. */
+int gern_hip_module_global(gern_hip_module module, const char *name, void **ptr, size_t *bytes);
+
 /* Device memory, for hosts that do not bring their own allocator (the
  * reference's data structures call cudaMalloc / cudaMemcpy themselves,
  * apps/common/impl/gpu-matrix-const.h:66-81,221-233). */

@@ -313,6 +313,52 @@ CASE("set_grid.block_size_from_own_variable_and_assumption") {
     set_grid_run(true);
 }
 
+// A kernel is compiled to rely on its launch assumptions, so one that the host cannot check
+// (the data structure does not say how to read the member it names) refuses the launch.
+namespace {
+class ArrayWithoutHostMembers : public annot::ArrayGPU {
+public:
+    using annot::ArrayGPU::ArrayGPU;
+    bool readMember(const void *, const std::string &, int64_t &) const override {
+        return false;
+    }
+};
+struct AddAssumingSize : annot::Add1GPU {
+    Annotation getAnnotation() override {
+        return resetUnit(annot::Add1GPU::getAnnotation(), {Grid::Unit::SCALAR_UNIT}).assumes(Constraint(output["size"] >= step));
+    }
+};
+}  // namespace
+
+CASE("set_grid.assumption_the_host_cannot_check_refuses_the_launch") {
+    for (bool readable : {true, false}) {
+        auto in = readable ? arrayDS("input_con") : AbstractDataTypePtr(new const ArrayWithoutHostMembers("input_con"));
+        auto out = readable ? arrayDS("output_con") : AbstractDataTypePtr(new const ArrayWithoutHostMembers("output_con"));
+        AddAssumingSize add_1;
+        Variable step("step");
+        Composable program = Global(Tile(out["size"], step)(add_1(in, out)));
+        Runner run(program);
+        if (!build(run, program)) {
+            return;
+        }
+        REQUIRE(last_source.find("__builtin_assume") != std::string::npos);
+        impl::ArrayGPU a(10), b(10);
+        a.ascending();
+        int64_t step_val = 5;
+        std::map<std::string, void *> args = {{in.getName(), &a}, {out.getName(), &b}, {step.getName(), &step_val}};
+        if (readable) {
+            REQUIRE_NOTHROW(run.evaluate(args));
+            expect_offset(a, b, 1, 10);
+            step_val = 20;  // violated
+            REQUIRE_THROWS_AS(run.evaluate(args), error::UserError);
+        } else {
+            REQUIRE_THROWS_AS(run.evaluate(args), error::UserError);
+        }
+        a.destroy();
+        b.destroy();
+    }
+}
+
 // ---- test-dynamic-shared.cu ----------------------------------------------------------------
 
 using annot::LdsManager;
@@ -488,6 +534,12 @@ CASE("schedule.gemm_staged_through_lds") {  // gernels/mm/kernel_3.cu:13-118 of 
         want00 += ha[kk] * hb[kk * n];
     }
     REQUIRE_EQ(got[0], 2 * want00);
+    REQUIRE_EQ(run.ldsOverflows(), 0);
+    // Too little dynamic LDS for both staged tiles (16 x 8 and 8 x 8 floats after the allocator's
+    // 128-byte table): the kernel still ends, and the host can tell that its results are void.
+    smem = 128 + 16 * 8 * 4 + 64;
+    run.evaluate({{A.getName(), &pa}, {B.getName(), &pb}, {C.getName(), &pc}, {smem_size.getName(), &smem}});
+    REQUIRE(run.ldsOverflows() > 0);
     a.destroy();
     b.destroy();
     c.destroy();
