@@ -6,19 +6,31 @@
 A step is one launch of the fused three-stage blur chain (x, y, x; 3 taps of
 weight 1/3) on an 8192 x 8192 fp32 image that is already resident in HBM; the
 headline value is its whole-job throughput in GB/s of ALGORITHMIC bytes
-(logical input read once + logical output written once).  The same line also
-carries the other configurations of the metric (row softmax, GEMM fp32 / bf16,
-fused QK^T softmax), each with its own roofline fraction, a roofline object
-for the dominant kernel timed with HIP events on the launching stream, and the
-CPU baseline: the reference library's own CPU lowering of the same composed
-pipeline (oracle/_ref/, when it was built) or the CPU oracle, timed on one host
-core.
+(logical input read once + logical output written once).
+
+The same line carries every other configuration of the metric under
+"workloads" (two-stage blur 1024^2, row softmax, GEMM fp32 / bf16, fused QK^T
+softmax, the user-level GEMM schedules at 1024^3).  Each entry holds the mean
+launch time over the timed steps, the median and minimum over at least 20
+launches timed one by one (HIP events on the launching stream), and its own
+"roofline" object: algorithmic bytes or flops per launch, the peak it is
+priced against, the fraction reached, and the HBM bytes per launch read from
+profiles/hbm_traffic.md -- used only when the kernel identity recorded there
+(a hash of the generated source and of the gernel headers) is the one that
+ran here; otherwise "traffic" is null and "traffic_note" says why.
+
+"cpu_baseline" is the reference library's own CPU lowering of the same
+composed pipeline (oracle/_ref/, when it was built) or the CPU oracle, timed
+on one host core.
 
 Prints exactly one JSON line on stdout.
 """
 import argparse
+import glob
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -28,12 +40,9 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA
-FP32_VECTOR_PEAK_TFLOPS = 157.3
-# HBM bytes one launch of the headline kernel moves, from the FETCH_SIZE and
-# WRITE_SIZE counters scaled by the plain-copy calibration kernel below
-# (profiles/bench_all_workloads_hbm_traffic.md).  Counters cannot be read from
-# inside this process; the figure is re-measured whenever the kernel changes.
-BLUR_XYX_8192_TRAFFIC_BYTES = 548743032
+FP32_PEAK_TFLOPS = 157.3       # fp32, matrix or packed vector
+MIN_SINGLE_LAUNCHES = 20
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.md")
 
 
 def log(*a):
@@ -65,6 +74,90 @@ def per_launch_ms(fn, n, torch, gern_amd):
         stop.record()
     torch.cuda.synchronize()
     return sorted(start.elapsed_ms_until(stop) for start, stop in pairs)
+
+
+DEVICE_WARMUP_S = 0.06
+
+
+def device_warmup(fn, torch):
+    """Untimed launches of the workload's own kernel for about 60 ms.  After idling (half a second
+    is enough) this GPU runs its first launches 10-25 % slower and takes some 25 ms of load to settle:
+    measured on the bf16 GEMM, 131-150 us per launch at first, 117 us from the 200th launch on."""
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < DEVICE_WARMUP_S or n == 0:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        n += 20
+    return n
+
+
+def measure(fn, warmup, steps, torch, gern_amd):
+    """Device warm-up, `warmup` more untimed launches, the mean over exactly `steps` back-to-back
+    launches, then median and minimum over single launches."""
+    device_warmup(fn, torch)
+    wall, ev = time_launches(fn, warmup, steps, torch, gern_amd)
+    n = max(MIN_SINGLE_LAUNCHES, min(steps, 50))
+    each = per_launch_ms(fn, n, torch, gern_amd)
+    return {"ms": ev, "wall_ms": wall, "steps": steps, "ms_median": each[len(each) // 2], "ms_min": each[0], "single_launches": n}
+
+
+_HEADER_HASH = []
+
+
+def kernel_id(source):
+    """Identity of a generated kernel: its source (the code generator numbers its functions per
+    process, so the number is masked) and every gernel header it may include."""
+    if not _HEADER_HASH:
+        h = hashlib.sha1()
+        for path in sorted(glob.glob(os.path.join(ROOT, "gern_amd", "gernels", "*.h"))):
+            with open(path, "rb") as f:
+                h.update(f.read())
+        _HEADER_HASH.append(h.hexdigest())
+    text = re.sub(r"function_\d+", "function_N", source)
+    return hashlib.sha1((text + _HEADER_HASH[0]).encode()).hexdigest()[:12]
+
+
+def traffic_table():
+    """Rows `| workload | kernel id | fetch bytes | write bytes |` of profiles/hbm_traffic.md."""
+    rows = {}
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 4 and re.fullmatch(r"[0-9a-f]{12}", cells[1]) and cells[2].isdigit() and cells[3].isdigit():
+                    rows[cells[0]] = (cells[1], int(cells[2]), int(cells[3]))
+    except OSError:
+        pass
+    return rows
+
+
+def roofline(workload, table, bound, algorithmic, timing, pipeline, source=None):
+    """bound "hbm": algorithmic bytes against 8 TB/s; "mfma" / "fp32": flops against the matrix peak."""
+    ms = timing["ms"]
+    if bound == "hbm":
+        achieved, peak, unit = algorithmic / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, unit = algorithmic / (ms * 1e-3) / 1e12, "TFLOP/s"
+        peak = MFMA_BF16_PEAK_TFLOPS if bound == "mfma" else FP32_PEAK_TFLOPS
+    kid = kernel_id(source if source is not None else pipeline.source)
+    roof = {"bound": "hbm" if bound == "hbm" else "mfma", "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+            "algorithmic": algorithmic, "algorithmic_unit": "bytes" if bound == "hbm" else "flop",
+            "kernel": pipeline.kernel_name, "kernel_id": kid, "kernel_ms": ms,
+            "kernel_ms_median": timing["ms_median"], "kernel_ms_min": timing["ms_min"],
+            "frac_at_median": achieved * ms / timing["ms_median"] / peak}
+    row = table.get(workload)
+    if row is None:
+        roof["traffic"] = None
+        roof["traffic_note"] = "no row for this workload in profiles/hbm_traffic.md"
+    elif row[0] != kid:
+        roof["traffic"] = None
+        roof["traffic_note"] = "the kernel changed since the counters were read (profiles/hbm_traffic.md has %s)" % row[0]
+    else:
+        roof["traffic"] = row[1] + row[2]
+        roof["traffic_fetch"], roof["traffic_write"] = row[1], row[2]
+    return roof
 
 
 COPY_SRC = r"""
@@ -105,43 +198,45 @@ def copy_calibration(torch, gern_amd, warmup, steps, kernel="gern_copy_f4", nbyt
     def launch():
         if hip.gern_hip_launch(ker, grid, block, 0, params, None) != 0:
             raise gern_amd.GernError(gern_amd._hip_error())
+    device_warmup(launch, torch)
     wall, ev = time_launches(launch, warmup, steps, torch, gern_amd)
     assert bool((dst == 1).all())
     return {"GB/s": 2 * nbytes / (ev * 1e-3) / 1e9, "ms": ev, "frac_hbm": 2 * nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "kernel": kernel, "bytes_read": nbytes, "bytes_written": nbytes}
 
 
-def cpu_baseline_blur(img_np):
-    """The same composed pipeline on ONE host core."""
+def cpu_blur(img_np, pattern, tile_rows, tile_cols, budget_s, what_size):
+    """The same composed pipeline on ONE host core: the reference library's CPU lowering when it
+    was built, else the CPU oracle with the same tiling."""
     from oracle import oracle as o
     from oracle import ref
     rows, cols = img_np.shape
     if ref.available():
         kind = "reference"
-        # tile sizes must divide the 8190 x 8188 output (the reference handles no ragged tiles)
-        run = lambda: ref.blur_chain(img_np, "xyx", 90, 356)  # noqa: E731
-        what = "reference library CPU lowering of Tile(rows=90)(Tile(cols=356)(blur_x, blur_y, blur_x)), g++ -O2"
+        run = lambda: ref.blur_chain(img_np, pattern, tile_rows, tile_cols)  # noqa: E731
+        what = "reference library CPU lowering of Tile(rows=%d)(Tile(cols=%d)(%s)), g++ -O2" % (
+            tile_rows, tile_cols, ", ".join("blur_" + c for c in pattern))
     else:
         kind = "port"
-        run = lambda: o.blur_chain_tiled(img_np, "xyx", 90, 356)  # noqa: E731
+        run = lambda: o.blur_chain_tiled(img_np, pattern, tile_rows, tile_cols)  # noqa: E731
         what = "CPU oracle (scalar C restatement), same tiling, gcc -O2"
-    run()  # warm-up
+    out = run()  # warm-up
     times = []
-    budget = time.perf_counter() + 20.0
+    budget = time.perf_counter() + budget_s
     while len(times) < 5 and (len(times) < 1 or time.perf_counter() < budget):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    nbytes = rows * cols * 4 + (rows - 2) * (cols - 4) * 4
-    return {
+    nbytes = img_np.nbytes + out.nbytes
+    return out, {
         "value": nbytes / med / 1e9,
         "unit": "GB/s",
         "cores": 1,
         "host_cores": os.cpu_count(),
         "kind": kind,
         "seconds": med,
-        "sample": "full workload (8192x8192 three-stage blur), median of %d runs after one warm-up; %s" % (len(times), what),
+        "sample": "full workload (%s), median of %d runs after one warm-up; %s" % (what_size, len(times), what),
     }
 
 
@@ -150,10 +245,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-rotating", action="store_true",
                     help="skip the extra timings over rotating buffers (profiles: keeps one kind of launch per kernel)")
-    ap.add_argument("--only", default="", help="run only this workload (blur, softmax, gemm_f32, gemm_bf16, qk_softmax, copy)")
+    ap.add_argument("--rotating-only", action="store_true",
+                    help="blur and softmax: time ONLY the launches over rotating buffers (counter runs of that regime)")
+    ap.add_argument("--only", default="", help="run only this workload (blur, blur_xy_1024, softmax, gemm_f32, gemm_bf16, "
+                                               "qk_softmax, gemm_schedules, copy)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -162,7 +260,7 @@ def main():
     import torch
 
     import __graft_entry__
-    __graft_entry__.ensure_built()  # builds only in a fresh checkout
+    __graft_entry__.ensure_built()
     import gern_amd
     from gern_amd import inputs
 
@@ -172,8 +270,21 @@ def main():
     log("device:", lim.arch.decode(), "CUs:", lim.compute_units)
 
     want = lambda name: (not args.only) or args.only == name  # noqa: E731
+    table = traffic_table()
     workloads = {}
     result = None
+    # every workload is timed over at least MIN_SINGLE_LAUNCHES launches, whatever --steps says
+    steps2 = max(MIN_SINGLE_LAUNCHES, args.steps // 4)
+    steps_gemm = max(MIN_SINGLE_LAUNCHES, args.steps // 10)
+
+    def rotating(pairs, launch):
+        turn = [0]
+
+        def fn():
+            a, b = pairs[turn[0] % len(pairs)]
+            turn[0] += 1
+            launch(a, b)
+        return fn
 
     # ---- config 2: three-stage blur, 8192 x 8192 (the headline) ------------
     if want("blur"):
@@ -182,94 +293,106 @@ def main():
         d_in = torch.from_numpy(img).cuda()
         blur = gern_amd.BlurChain("xyx", tile_rows=4)  # 4 x 224 tiles, line-aligned store windows
         d_out = torch.zeros(blur.out_shape(rows, cols), device="cuda")
-        wall, ev = time_launches(lambda: blur(d_in, d_out), args.warmup, args.steps, torch, gern_amd)
         nbytes = img.nbytes + d_out.numel() * 4
-        gbs = nbytes / (wall * 1e-3) / 1e9
-        roof = {"bound": "hbm", "achieved": nbytes / (ev * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": BLUR_XYX_8192_TRAFFIC_BYTES,
-                "kernel": blur.kernel_name, "kernel_ms": ev, "algorithmic_bytes": nbytes}
-        each = per_launch_ms(lambda: blur(d_in, d_out), 50, torch, gern_amd)
-        roof["kernel_ms_median"] = each[len(each) // 2]
-        roof["kernel_ms_min"] = each[0]
-        workloads["blur_xyx_8192"] = {"GB/s": gbs, "ms": wall, "frac_hbm": gbs / HBM_PEAK_GBS}
-        log("blur xyx 8192^2: %.1f us/launch  %.0f GB/s  (%.1f%% of HBM peak)" % (wall * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
+        if not args.rotating_only:
+            t = measure(lambda: blur(d_in, d_out), args.warmup, args.steps, torch, gern_amd)
+            gbs = nbytes / (t["wall_ms"] * 1e-3) / 1e9
+            roof = roofline("blur_xyx_8192", table, "hbm", nbytes, t, blur)
+            workloads["blur_xyx_8192"] = {"GB/s": gbs, "ms": t["wall_ms"], "frac_hbm": gbs / HBM_PEAK_GBS, "roofline": roof}
+            log("blur xyx 8192^2: %.1f us/launch  %.0f GB/s  (%.1f%% of HBM peak)" % (t["wall_ms"] * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
         if not args.no_rotating:
             # The same launch over ROTATING buffer pairs: the 256 MiB image is exactly the size of the
             # memory-side cache, and with streaming stores a launch finds part of its input there when
             # the previous launch read the same buffer.  Rotating over four pairs takes that away.
             ring = [(d_in, d_out)] + [(d_in.clone(), torch.zeros_like(d_out)) for _ in range(3)]
-            turn = [0]
-
-            def rotating():
-                a, b = ring[turn[0] % len(ring)]
-                turn[0] += 1
-                blur(a, b)
-            wall_r, ev_r = time_launches(rotating, args.warmup, args.steps, torch, gern_amd)
-            workloads["blur_xyx_8192_rotating_buffers"] = {"GB/s": nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
-                                                           "frac_hbm": nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS, "buffer_pairs": len(ring)}
-            log("blur xyx 8192^2 over %d rotating buffer pairs: %.1f us/launch  %.0f GB/s" % (len(ring), ev_r * 1e3, nbytes / (ev_r * 1e-3) / 1e9))
-            # `value`, `achieved` and `frac` follow the reference's own protocol (apps/blur/blur.cu:79-96: warm-up,
-            # then N launches on the SAME buffers); the rotating figure is what HBM alone sustains.
-            roof["achieved_rotating_buffers"] = nbytes / (ev_r * 1e-3) / 1e9
-            roof["frac_rotating_buffers"] = roof["achieved_rotating_buffers"] / HBM_PEAK_GBS
-            roof["kernel_ms_rotating_buffers"] = ev_r
+            tr = measure(rotating(ring, lambda a, b: blur(a, b)), args.warmup, args.steps, torch, gern_amd)
+            rroof = roofline("blur_xyx_8192_rotating_buffers", table, "hbm", nbytes, tr, blur)
+            workloads["blur_xyx_8192_rotating_buffers"] = {"GB/s": rroof["achieved"], "ms": tr["ms"], "frac_hbm": rroof["frac"],
+                                                           "buffer_pairs": len(ring), "roofline": rroof}
+            log("blur xyx 8192^2 over %d rotating buffer pairs: %.1f us/launch  %.0f GB/s" % (len(ring), tr["ms"] * 1e3, rroof["achieved"]))
             del ring
-        result = {
-            "metric": "fused 3-stage blur (x,y,x) 8192x8192 fp32, algorithmic GB/s",
-            "value": gbs,
-            "unit": "GB/s",
-            "n_gpus": 1,
-            "steps": args.steps,
-            "warmup": args.warmup,
-            "ms_per_step": wall,
-            "higher_is_better": True,
-            "scaling": "weak",
-            "vs_baseline": None,
-            "dtype": "f32",
-            "data": "synthetic",
-            "config": {"workload": "three-stage fused separable blur chain (3-tap x, y, x; weights 1/3), 8192x8192 fp32 "
-                                   "uniform[0,1) seed 2, valid-region output 8190x8188, one launch per step",
-                       "schedule": "one wavefront per 4x224 output tile, store windows moved to whole 128-byte lines, XCD-aware workgroup order",
-                       "protocol": "the reference's: warm-up, then `steps` launches on the same buffers "
-                                   "(roofline.achieved_rotating_buffers: the same launches over four rotating "
-                                   "buffer pairs, which takes the 256 MiB memory-side cache out of the figure)"},
-            "roofline": roof,
-        }
-        if not args.no_cpu:
-            result["cpu_baseline"] = cpu_baseline_blur(img)
-            log("cpu baseline: %.2f GB/s on 1 core (%s)" % (result["cpu_baseline"]["value"], result["cpu_baseline"]["kind"]))
+        if not args.rotating_only:
+            if not args.no_rotating:
+                # `value`, `achieved` and `frac` follow the reference's own protocol (apps/blur/blur.cu:79-96: warm-up,
+                # then N launches on the SAME buffers); the rotating figure is what HBM alone sustains.
+                roof["achieved_rotating_buffers"] = rroof["achieved"]
+                roof["frac_rotating_buffers"] = rroof["frac"]
+                roof["kernel_ms_rotating_buffers"] = tr["ms"]
+                roof["traffic_rotating_buffers"] = rroof["traffic"]
+            result = {
+                "metric": "fused 3-stage blur (x,y,x) 8192x8192 fp32, algorithmic GB/s",
+                "value": gbs,
+                "unit": "GB/s",
+                "n_gpus": 1,
+                "steps": args.steps,
+                "warmup": args.warmup,
+                "ms_per_step": t["wall_ms"],
+                "higher_is_better": True,
+                "scaling": "weak",
+                "vs_baseline": None,
+                "dtype": "f32",
+                "data": "synthetic",
+                "config": {"workload": "three-stage fused separable blur chain (3-tap x, y, x; weights 1/3), 8192x8192 fp32 "
+                                       "uniform[0,1) seed 2, valid-region output 8190x8188, one launch per step",
+                           "schedule": "one wavefront per 4x224 output tile, store windows moved to whole 128-byte lines, "
+                                       "XCD-aware workgroup order",
+                           "protocol": "about 60 ms of untimed launches (the GPU settles), `warmup` more untimed launches, then, as "
+                                       "the reference does, `steps` timed launches on the same buffers "
+                                       "(roofline.achieved_rotating_buffers: the same launches over four rotating "
+                                       "buffer pairs, which takes the 256 MiB memory-side cache out of the figure)"},
+                "roofline": roof,
+            }
+            if not args.no_cpu:
+                # tile sizes must divide the 8190 x 8188 output (the reference handles no ragged tiles)
+                _, result["cpu_baseline"] = cpu_blur(img, "xyx", 90, 356, 20.0, "8192x8192 three-stage blur")
+                log("cpu baseline: %.2f GB/s on 1 core (%s)" % (result["cpu_baseline"]["value"], result["cpu_baseline"]["kind"]))
         del d_in, d_out
 
-    steps2 = max(10, args.steps // 4)
+    # ---- config 1: two-stage blur, 1024 x 1024 (the reference's CPU-runnable case) ----
+    if want("blur_xy_1024") and not args.rotating_only:
+        img = inputs.uniform((1024, 1024), 1)
+        d_in = torch.from_numpy(img).cuda()
+        blur = gern_amd.BlurChain("xy")
+        d_out = torch.zeros(blur.out_shape(1024, 1024), device="cuda")
+        nbytes = img.nbytes + d_out.numel() * 4
+        t = measure(lambda: blur(d_in, d_out), args.warmup, steps2, torch, gern_amd)
+        roof = roofline("blur_xy_1024", table, "hbm", nbytes, t, blur)
+        workloads["blur_xy_1024"] = {"GB/s": roof["achieved"], "ms": t["ms"], "frac_hbm": roof["frac"], "roofline": roof,
+                                     "note": "8 MB of traffic: launch latency, not HBM, bounds a launch this small"}
+        log("blur xy 1024^2: %.1f us  %.0f GB/s" % (t["ms"] * 1e3, roof["achieved"]))
+        if not args.no_cpu:
+            # 1022 x 1022 output = (14 x 73) x (7 x 146) tiles
+            want_out, cpu = cpu_blur(img, "xy", 73, 146, 5.0, "1024x1024 two-stage blur")
+            torch.cuda.synchronize()
+            cpu["gpu_result_identical"] = bool(np.array_equal(d_out.cpu().numpy(), want_out))
+            workloads["blur_xy_1024_cpu"] = cpu
+            log("blur xy 1024^2 on the CPU: %.2f GB/s on 1 core (%s), GPU result identical: %s" % (cpu["value"], cpu["kind"], cpu["gpu_result_identical"]))
+        del d_in, d_out
+
     # ---- config 3: row softmax, 8192 x 4096 --------------------------------
     if want("softmax"):
         x = inputs.normal((8192, 4096), 3, 0.0, 2.0)
         d_x = torch.from_numpy(x).cuda()
         d_y = torch.zeros_like(d_x)
         sm = gern_amd.Softmax(4096)
-        wall, ev = time_launches(lambda: sm(d_x, d_y), args.warmup, steps2, torch, gern_amd)
-        gbs = 2 * x.nbytes / (ev * 1e-3) / 1e9
-        workloads["softmax_8192x4096"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "kernel": sm.kernel_name}
-        log("softmax 8192x4096: %.1f us  %.0f GB/s (%.1f%%)" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS))
+        if not args.rotating_only:
+            t = measure(lambda: sm(d_x, d_y), args.warmup, steps2, torch, gern_amd)
+            roof = roofline("softmax_8192x4096", table, "hbm", 2 * x.nbytes, t, sm)
+            workloads["softmax_8192x4096"] = {"GB/s": roof["achieved"], "ms": t["ms"], "frac_hbm": roof["frac"], "roofline": roof}
+            log("softmax 8192x4096: %.1f us  %.0f GB/s (%.1f%%)" % (t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"]))
         if not args.no_rotating:
             ring = [(d_x, d_y)] + [(d_x.clone(), torch.zeros_like(d_y)) for _ in range(5)]
-            turn = [0]
-
-            def rotating_softmax():
-                a, b = ring[turn[0] % len(ring)]
-                turn[0] += 1
-                sm(a, b)
-            wall_r, ev_r = time_launches(rotating_softmax, args.warmup, steps2, torch, gern_amd)
-            workloads["softmax_8192x4096_rotating_buffers"] = {"GB/s": 2 * x.nbytes / (ev_r * 1e-3) / 1e9, "ms": ev_r,
-                                                               "frac_hbm": 2 * x.nbytes / (ev_r * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                                                               "buffer_pairs": len(ring)}
-            log("softmax 8192x4096 over %d rotating buffer pairs: %.1f us  %.0f GB/s" % (len(ring), ev_r * 1e3, 2 * x.nbytes / (ev_r * 1e-3) / 1e9))
+            tr = measure(rotating(ring, lambda a, b: sm(a, b)), args.warmup, steps2, torch, gern_amd)
+            rroof = roofline("softmax_8192x4096_rotating_buffers", table, "hbm", 2 * x.nbytes, tr, sm)
+            workloads["softmax_8192x4096_rotating_buffers"] = {"GB/s": rroof["achieved"], "ms": tr["ms"], "frac_hbm": rroof["frac"],
+                                                               "buffer_pairs": len(ring), "roofline": rroof}
+            log("softmax 8192x4096 over %d rotating buffer pairs: %.1f us  %.0f GB/s" % (len(ring), tr["ms"] * 1e3, rroof["achieved"]))
             del ring
         del d_x, d_y
 
     # ---- config 4: GEMM 4096^3 ---------------------------------------------
-    for variant, peak in (("f32", FP32_VECTOR_PEAK_TFLOPS), ("bf16", MFMA_BF16_PEAK_TFLOPS)):
-        if not want("gemm_" + variant):
+    for variant, bound in (("f32", "fp32"), ("bf16", "mfma")):
+        if not want("gemm_" + variant) or args.rotating_only:
             continue
         n = 4096
         A = inputs.uniform((n, n), 4, -1.0, 1.0)
@@ -281,23 +404,24 @@ def main():
             dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
         dC = torch.zeros((n, n), device="cuda")
         g = gern_amd.Gemm(variant, overwrite=True)  # config 4 is C = A * B
-        wall, ev = time_launches(lambda: g(dA, dB, dC), 3, max(5, args.steps // 20), torch, gern_amd)
-        tf = 2.0 * n ** 3 / (ev * 1e-3) / 1e12
-        workloads["gemm_%s_4096" % variant] = {"TFLOP/s": tf, "ms": ev, "frac_peak": tf / peak, "peak_TFLOP/s": peak,
-                                               "kernel": g.kernel_name}
-        log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, ev * 1e3, tf, 100 * tf / peak, peak))
+        t = measure(lambda: g(dA, dB, dC), 5, steps_gemm, torch, gern_amd)
+        roof = roofline("gemm_%s_4096" % variant, table, bound, 2.0 * n ** 3, t, g)
+        workloads["gemm_%s_4096" % variant] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
+                                               "peak_TFLOP/s": roof["peak"], "roofline": roof}
+        log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], roof["peak"]))
         if variant == "f32":
             # the same product on the kernel that takes every shape (vector-ALU FMAs)
             g = gern_amd.Gemm(variant, overwrite=True, general_only=True)
-            wall, ev = time_launches(lambda: g(dA, dB, dC), 3, max(5, args.steps // 20), torch, gern_amd)
-            tf = 2.0 * n ** 3 / (ev * 1e-3) / 1e12
-            workloads["gemm_f32_4096_vector_alu"] = {"TFLOP/s": tf, "ms": ev, "frac_peak": tf / peak, "peak_TFLOP/s": peak,
-                                                     "kernel": g.kernel_name}
-            log("gemm f32 4096^3, vector-ALU kernel: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (ev * 1e3, tf, 100 * tf / peak, peak))
+            t = measure(lambda: g(dA, dB, dC), 3, steps_gemm, torch, gern_amd)
+            roof = roofline("gemm_f32_4096_vector_alu", table, bound, 2.0 * n ** 3, t, g)
+            workloads["gemm_f32_4096_vector_alu"] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
+                                                     "peak_TFLOP/s": roof["peak"], "roofline": roof}
+            log("gemm f32 4096^3, vector-ALU kernel: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (
+                t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], roof["peak"]))
         del dA, dB, dC
 
     # ---- config 5: fused QK^T -> softmax ------------------------------------
-    if want("qk_softmax"):
+    if want("qk_softmax") and not args.rotating_only:
         m = nk = 4096
         d = 128
         Q = inputs.to_bf16_bits(inputs.normal((m, d), 5))
@@ -307,16 +431,35 @@ def main():
         dS = torch.zeros((m, nk), device="cuda")
         qk = gern_amd.QKSoftmax(d, nk)
         scale = 1.0 / np.sqrt(float(d))
-        wall, ev = time_launches(lambda: qk(dQ, dK, dS, scale), args.warmup, steps2, torch, gern_amd)
+        t = measure(lambda: qk(dQ, dK, dS, scale), args.warmup, steps2, torch, gern_amd)
         nbytes = Q.nbytes + K.nbytes + m * nk * 4
-        gbs = nbytes / (ev * 1e-3) / 1e9
-        tf = 2.0 * m * nk * d / (ev * 1e-3) / 1e12
-        workloads["qk_softmax_4096x4096x128"] = {"GB/s": gbs, "ms": ev, "frac_hbm": gbs / HBM_PEAK_GBS, "TFLOP/s": tf,
-                                                 "frac_mfma": tf / MFMA_BF16_PEAK_TFLOPS, "kernel": qk.kernel_name}
-        log("qk softmax 4096x4096x128: %.1f us  %.0f GB/s (%.1f%% HBM)  %.1f TFLOP/s" % (ev * 1e3, gbs, 100 * gbs / HBM_PEAK_GBS, tf))
+        roof = roofline("qk_softmax_4096x4096x128", table, "hbm", nbytes, t, qk)
+        tf = 2.0 * m * nk * d / (t["ms"] * 1e-3) / 1e12
+        workloads["qk_softmax_4096x4096x128"] = {"GB/s": roof["achieved"], "ms": t["ms"], "frac_hbm": roof["frac"], "TFLOP/s": tf,
+                                                 "frac_mfma": tf / MFMA_BF16_PEAK_TFLOPS, "roofline": roof}
+        log("qk softmax 4096x4096x128: %.1f us  %.0f GB/s (%.1f%% HBM)  %.1f TFLOP/s" % (t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], tf))
+        del dQ, dK, dS
+
+    # ---- schedules written at the level of Gern's API, 1024^3 (the reference times such a
+    # kernel in gernels/mm/bench.cu:72-89) ---------------------------------------------------
+    if want("gemm_schedules") and not args.rotating_only:
+        n = gern_amd.GemmSchedule.SIZE
+        dA = torch.from_numpy(inputs.uniform((n, n), 4, -1.0, 1.0)).cuda()
+        dB = torch.from_numpy(inputs.uniform((n, n), 5, -1.0, 1.0)).cuda()
+        dC = torch.zeros((n, n), device="cuda")
+        for schedule, what in ((3, "block tiles staged through LDS one float per lane, 4x4 outputs per thread"),
+                               (6, "staged 16 bytes per lane"),
+                               (10, "block -> wavefront -> lane tiling, loads that write LDS directly, one output per lane")):
+            g = gern_amd.GemmSchedule(schedule)
+            t = measure(lambda: g(dA, dB, dC), 3, MIN_SINGLE_LAUNCHES, torch, gern_amd)
+            roof = roofline("gemm_schedule_kernel_%d_1024" % schedule, table, "fp32", 2.0 * n ** 3, t, g)
+            workloads["gemm_schedule_kernel_%d_1024" % schedule] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
+                                                                    "schedule": what, "roofline": roof}
+            log("gemm schedule kernel_%d 1024^3: %.1f us  %.2f TFLOP/s" % (schedule, t["ms"] * 1e3, roof["achieved"]))
+        del dA, dB, dC
 
     # ---- calibration: plain copy of known size ------------------------------
-    if want("copy"):
+    if want("copy") and not args.rotating_only:
         workloads["copy_256MiB"] = copy_calibration(torch, gern_amd, args.warmup, steps2)
         log("copy 256 MiB: %.1f us  %.0f GB/s" % (workloads["copy_256MiB"]["ms"] * 1e3, workloads["copy_256MiB"]["GB/s"]))
         workloads["copy_256MiB_streaming_stores"] = copy_calibration(torch, gern_amd, args.warmup, steps2,
@@ -331,7 +474,8 @@ def main():
                                                                      workloads["copy_1GiB_streaming_stores"]["GB/s"]))
 
     if result is None:
-        result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "", "n_gpus": 1,
+        result = {"metric": "partial run (--only %s%s)" % (args.only, " --rotating-only" if args.rotating_only else ""),
+                  "value": None, "unit": "", "n_gpus": 1,
                   "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
                   "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": args.only}}
     result["workloads"] = workloads

@@ -21,6 +21,7 @@ GEMM_OVERWRITE = 4
 GEMM_GENERAL_ONLY = 8
 BLUR_PLAIN_STORES = 16
 QK_ROW_BLOCKS = 32
+XCD_TILE_BLOCKS = 64
 
 _libs = None
 

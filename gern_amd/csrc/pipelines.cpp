@@ -96,6 +96,7 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
         if (flags & GERN_PIPELINE_COMPILE_ONLY) {
             codegen::GeneratorOptions go;
             go.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+            go.xcd_tile_blocks = (flags & GERN_PIPELINE_XCD_TILE_BLOCKS) != 0;
             go.min_waves_per_simd = min_waves_per_simd;
             codegen::CodeGenerator cg(std::nullopt, go);
             p->source = cg.generate_code(program);
@@ -128,6 +129,7 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
         options.filename = "";  // keep the source in memory only
         options.include = include;
         options.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+        options.xcd_tile_blocks = (flags & GERN_PIPELINE_XCD_TILE_BLOCKS) != 0;
         options.min_waves_per_simd = min_waves_per_simd;
         p->runner->compile(options);
         p->source = p->runner->getSource();
@@ -377,6 +379,11 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
         // XCD's L2.  Giving each XCD a contiguous band of ids (the renumbering that
         // helps the blur) makes that block one tile row of many columns: at 8192^3,
         // 33 panels per 32 tiles instead of 12, and 6 % slower (measured).
+        // The kernels therefore take the order that makes the block explicit: 4 x 8 tiles per XCD at a
+        // time, 12 panels per 32 tiles (at 4096^3 the plain order gives 2 x 16 tiles of 256 x 256, 18 panels).
+        if (!(flags & GERN_PIPELINE_NO_XCD_REMAP)) {
+            flags |= GERN_PIPELINE_XCD_TILE_BLOCKS;
+        }
         flags |= GERN_PIPELINE_NO_XCD_REMAP;
         // The kernel for every shape.  bf16: four wavefronts, 256x256 tile, LDS of
         // gernels/mm.h mfma_lds_bytes(); fp32: vector-ALU FMAs, 128x128 tile, LDS

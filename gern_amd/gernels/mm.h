@@ -413,19 +413,29 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         __builtin_amdgcn_s_barrier();
     };
 
+    // Diagnostic builds only (gern_amd.microbench, results are wrong): -DGERN_MM_ONLY=1 moves the
+    // data and computes nothing, -DGERN_MM_ONLY=2 computes every stage on what the first two loaded.
+#ifndef GERN_MM_ONLY
+#define GERN_MM_ONLY 0
+#endif
+    constexpr bool kCompute = GERN_MM_ONLY != 1, kReload = GERN_MM_ONLY != 2;
     issue(0, stage_even);
     arrive();
     for (int kt = 0; kt < nk; kt += 2) {
-        if (kt + 1 < nk) {
+        if (kt + 1 < nk && (kReload || kt == 0)) {
             issue(kt + 1, stage_odd);
         }
-        compute(stage_even);
+        if (kCompute) {
+            compute(stage_even);
+        }
         arrive();
         if (kt + 1 < nk) {
-            if (kt + 2 < nk) {
+            if (kt + 2 < nk && kReload) {
                 issue(kt + 2, stage_even);
             }
-            compute(stage_odd);
+            if (kCompute) {
+                compute(stage_odd);
+            }
             arrive();
         }
     }

@@ -55,6 +55,8 @@ bool evaluate(const Constraint &c, const EvalEnv &env, bool &value);
 
 struct GeneratorOptions {
     bool xcd_remap = true;
+    // Instead: each XCD takes blocks of 4 x 8 tiles (see Runner::Options).
+    bool xcd_tile_blocks = false;
     // Wavefronts per SIMD the kernel must leave room for (second argument of
     // __launch_bounds__): caps its registers at 512 / n.  0 = the compiler decides.
     int min_waves_per_simd = 0;

@@ -42,6 +42,12 @@ public:
         // Spread consecutive workgroups of one XCD over neighbouring tiles
         // (each of the 8 XCDs of an MI355X has its own L2).
         bool xcd_remap = true;
+        // Instead of that: the 32 workgroups that run on one XCD at a time take a
+        // block of 4 x 8 tiles (x by y), for programs whose tiles share operands
+        // along both grid axes (a GEMM: 12 operand panels per 32 tiles).  Applies
+        // to launches whose grid is a multiple of 4 by 8 workgroups with a multiple
+        // of 256 of them per z slice; other launches keep the plain order.
+        bool xcd_tile_blocks = false;
         // Wavefronts per SIMD the kernel must leave room for (caps its
         // registers at 512 / n); 0 = the compiler decides.
         int min_waves_per_simd = 0;

@@ -2,13 +2,19 @@
 """In-kernel clocks of the matrix-core pipelines, and the machine rates they are
 judged against, on ONE MI355X.
 
-    python -m gern_amd.microbench [gemm_bf16_phases] [qk_phases] [mfma_rate] [write_rate]
+    python -m gern_amd.microbench [gemm_bf16_phases] [gemm_bf16_split] [vendor_gemm] [qk_phases] [mfma_rate] [write_rate]
 
 gemm_bf16_phases  the bf16 GEMM 4096^3 kernel as the code generator emits it
                   (same gernel calls, gernels/mm.h), with the 100 MHz
                   wall clock and the shader clock read by every workgroup
                   before the K loop, after it, after its stores are issued and
                   after they are acknowledged
+gemm_bf16_split   the bf16 GEMM 4096^3 and 8192^3 pipeline built three ways and timed
+                  in turn in one process: as it is, moving the data only (no LDS
+                  reads, no MFMAs), and computing only (every stage on what the
+                  first two loaded)
+vendor_gemm       torch.matmul (the vendor's GEMM library) on the same shapes,
+                  bf16 and fp32: what tuned code of the vendor reaches on this GPU
 qk_phases         the same for the QK^T softmax tile kernel (gernels/qk_tiles.h)
 mfma_rate         a loop of nothing but v_mfma_f32_32x32x16_bf16 with changing
                   operands on every SIMD for about a millisecond: the sustained
@@ -223,6 +229,59 @@ def gemm_bf16_phases(gern_amd, torch):
     print("  2 * 4096^3 flop / per-launch time = %.0f TFLOP/s" % (2.0 * n ** 3 / (us * 1e-6) / 1e12))
 
 
+def gemm_bf16_split(gern_amd, torch):
+    from gern_amd import inputs
+    for n in (4096, 8192):
+        A = inputs.to_bf16_bits(inputs.uniform((n, n), 4, -1.0, 1.0))
+        B = inputs.to_bf16_bits(inputs.uniform((n, n), 5, -1.0, 1.0))
+        dA, dB = torch.from_numpy(A.view(np.int16)).cuda(), torch.from_numpy(B.view(np.int16)).cuda()
+        dC = torch.zeros((n, n), device="cuda")
+        builds = [("as it is", ""), ("data movement only", "-DGERN_MM_ONLY=1"), ("compute only", "-DGERN_MM_ONLY=2")]
+        pipes = []
+        before = os.environ.get("GERN_PIPELINE_EXTRA_OPTIONS")
+        for _, opt in builds:
+            os.environ["GERN_PIPELINE_EXTRA_OPTIONS"] = ((before or "") + " " + opt).strip()
+            pipes.append(gern_amd.Gemm("bf16", overwrite=True))
+        if before is None:
+            del os.environ["GERN_PIPELINE_EXTRA_OPTIONS"]
+        else:
+            os.environ["GERN_PIPELINE_EXTRA_OPTIONS"] = before
+        times = [[] for _ in builds]
+        for _ in range(100):
+            pipes[0](dA, dB, dC)
+        for rep in range(5):
+            for i, p in enumerate(pipes):
+                times[i].append(_event_us(gern_amd, torch, lambda: p(dA, dB, dC), 5, 30))
+        print("bf16 GEMM %d^3, whole-tile kernel, three builds timed in turn (us per launch, 5 rounds of 30 launches):" % n)
+        for (name, _), t in zip(builds, times):
+            print("  %-20s %s   min %.1f us = %.0f TFLOP/s-equivalent" % (name + ":", " ".join("%.1f" % x for x in t), min(t),
+                                                                          2.0 * n ** 3 / (min(t) * 1e-6) / 1e12))
+        del pipes
+
+
+def vendor_gemm(gern_amd, torch):
+    print("torch.matmul (vendor GEMM library), uniform [-1, 1) operands, us per launch over 5 rounds of 30 launches:")
+    for n in (4096, 8192):
+        for dt, name in ((torch.bfloat16, "bf16"), (torch.float32, "fp32")):
+            A = (torch.rand(n, n, device="cuda") * 2 - 1).to(dt)
+            B = (torch.rand(n, n, device="cuda") * 2 - 1).to(dt)
+            out = torch.empty(n, n, device="cuda", dtype=dt)
+            for _ in range(10):
+                torch.matmul(A, B, out=out)
+            torch.cuda.synchronize()
+            res = []
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(30):
+                    torch.matmul(A, B, out=out)
+                e1.record()
+                torch.cuda.synchronize()
+                res.append(e0.elapsed_time(e1) / 30 * 1e3)
+            print("  %d^3 %s: %s   min %.1f us = %.0f TFLOP/s" % (n, name, " ".join("%.1f" % r for r in res), min(res),
+                                                                   2.0 * n ** 3 / (min(res) * 1e-6) / 1e12))
+
+
 def qk_phases(gern_amd, torch):
     from gern_amd import inputs
     m = n = 4096
@@ -284,7 +343,7 @@ def main():
     import gern_amd
     if gern_amd.device_count() < 1 or not torch.cuda.is_available():
         sys.exit("gern_amd.microbench needs a GPU")
-    probes = {"gemm_bf16_phases": gemm_bf16_phases, "qk_phases": qk_phases, "mfma_rate": mfma_rate, "write_rate": write_rate}
+    probes = {"gemm_bf16_phases": gemm_bf16_phases, "gemm_bf16_split": gemm_bf16_split, "vendor_gemm": vendor_gemm, "qk_phases": qk_phases, "mfma_rate": mfma_rate, "write_rate": write_rate}
     chosen = sys.argv[1:] or list(probes)
     for name in chosen:
         if name not in probes:

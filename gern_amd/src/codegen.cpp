@@ -295,13 +295,13 @@ public:
         switch (u) {
         case Grid::BLOCK_X:
             uses_block_units = true;
-            return options.xcd_remap ? "gern_block_x" : "blockIdx.x";
+            return (options.xcd_remap || options.xcd_tile_blocks) ? "gern_block_x" : "blockIdx.x";
         case Grid::BLOCK_Y:
             uses_block_units = true;
-            return options.xcd_remap ? "gern_block_y" : "blockIdx.y";
+            return (options.xcd_remap || options.xcd_tile_blocks) ? "gern_block_y" : "blockIdx.y";
         case Grid::BLOCK_Z:
             uses_block_units = true;
-            return options.xcd_remap ? "gern_block_z" : "blockIdx.z";
+            return (options.xcd_remap || options.xcd_tile_blocks) ? "gern_block_z" : "blockIdx.z";
         case Grid::THREAD_X:
             return "threadIdx.x";
         case Grid::THREAD_Y:
@@ -589,7 +589,25 @@ std::string CodeGenerator::generate_code(Composable c) {
         out << (i ? ", " : "") << p.getType() << ((device || !p.isData()) ? " " : " &") << name;
     }
     out << ") {\n";
-    if (device && em.uses_block_units && options.xcd_remap) {
+    if (device && em.uses_block_units && options.xcd_tile_blocks) {
+        // Workgroups are handed to the 8 XCDs round-robin in launch order, so
+        // the l-th workgroup of XCD x has launch number 8 l + x.  The 32 that
+        // an XCD runs at a time (one per CU) take a block of 4 x 8 tiles:
+        // block number (l / 32) * 8 + x, tile l % 32 inside it.
+        out << "    const unsigned gern_nbx = gridDim.x, gern_nby = gridDim.y;\n"
+               "    unsigned gern_bx = blockIdx.x, gern_by = blockIdx.y;\n"
+               "    if (gern_nbx % 4u == 0u && gern_nby % 8u == 0u && (gern_nbx * gern_nby) % 256u == 0u) {\n"
+               "        const unsigned gern_wg = blockIdx.x + gern_nbx * blockIdx.y;\n"
+               "        const unsigned gern_l = gern_wg / 8u;\n"
+               "        const unsigned gern_sb = (gern_l / 32u) * 8u + gern_wg % 8u;\n"
+               "        gern_bx = (gern_sb % (gern_nbx / 4u)) * 4u + gern_l % 4u;\n"
+               "        gern_by = (gern_sb / (gern_nbx / 4u)) * 8u + (gern_l % 32u) / 4u;\n"
+               "    }\n"
+               "    const int64_t gern_block_x = gern_bx;\n"
+               "    const int64_t gern_block_y = gern_by;\n"
+               "    const int64_t gern_block_z = blockIdx.z;\n"
+               "    (void)gern_block_x; (void)gern_block_y; (void)gern_block_z;\n";
+    } else if (device && em.uses_block_units && options.xcd_remap) {
         // Workgroups are handed to the 8 XCDs round-robin in launch order.
         // Renumbering them so that each XCD walks a contiguous run of tiles
         // keeps halo and shared-line traffic inside one XCD's L2.

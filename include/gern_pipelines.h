@@ -47,7 +47,13 @@ enum {
     GERN_PIPELINE_BLUR_PLAIN_STORES = 16,
     /* QK^T softmax only: sixteen whole rows of S per workgroup also for head
      * dimensions that the 256 x 256 tile kernel takes (multiples of 64). */
-    GERN_PIPELINE_QK_ROW_BLOCKS = 32
+    GERN_PIPELINE_QK_ROW_BLOCKS = 32,
+    /* Workgroup order in which the 32 workgroups that run on one XCD at a
+     * time take a block of 4 x 8 tiles (grids that are a multiple of 4 x 8
+     * workgroups and of 256 in all; others keep the plain order).  The
+     * matrix-core GEMM kernels use it unless GERN_PIPELINE_NO_XCD_REMAP asks
+     * for the plain order. */
+    GERN_PIPELINE_XCD_TILE_BLOCKS = 64
 };
 
 /* Device memory through which the workgroups of the QK^T softmax tile kernel
