@@ -107,15 +107,15 @@ _HEADER_HASH = []
 
 
 def kernel_id(source):
-    """Identity of a generated kernel: its source (the code generator numbers its functions per
-    process, so the number is masked) and every gernel header it may include."""
+    """Identity of a generated kernel: its source (the code generator numbers functions and variables
+    per process, so trailing numbers of identifiers are masked) and every gernel header it may include."""
     if not _HEADER_HASH:
         h = hashlib.sha1()
         for path in sorted(glob.glob(os.path.join(ROOT, "gern_amd", "gernels", "*.h"))):
             with open(path, "rb") as f:
                 h.update(f.read())
         _HEADER_HASH.append(h.hexdigest())
-    text = re.sub(r"function_\d+", "function_N", source)
+    text = re.sub(r"(?:_\d+)+\b", "_N", source)
     return hashlib.sha1((text + _HEADER_HASH[0]).encode()).hexdigest()[:12]
 
 
@@ -250,7 +250,7 @@ def main():
                     help="skip the extra timings over rotating buffers (profiles: keeps one kind of launch per kernel)")
     ap.add_argument("--rotating-only", action="store_true",
                     help="blur and softmax: time ONLY the launches over rotating buffers (counter runs of that regime)")
-    ap.add_argument("--only", default="", help="run only this workload (blur, blur_xy_1024, softmax, gemm_f32, gemm_bf16, "
+    ap.add_argument("--only", default="", help="run only these workloads, comma-separated (blur, blur_xy_1024, softmax, gemm_f32, gemm_bf16, "
                                                "qk_softmax, gemm_schedules, copy)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -269,7 +269,8 @@ def main():
     lim = gern_amd.device_limits()
     log("device:", lim.arch.decode(), "CUs:", lim.compute_units)
 
-    want = lambda name: (not args.only) or args.only == name  # noqa: E731
+    only = [w for w in args.only.split(",") if w]
+    want = lambda name: (not only) or name in only  # noqa: E731
     table = traffic_table()
     workloads = {}
     result = None

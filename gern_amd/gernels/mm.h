@@ -544,12 +544,16 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_
         }
     };
 
-    // Workgroups that run at the same time start their walk over K at
-    // different steps (and wrap around).  With a power-of-two row pitch the
-    // rows of one K step all fall into the same memory channel; if every
-    // workgroup asked for the same step at once, one channel would serve the
-    // whole chip.  The sum over K does not depend on where the walk starts.
-    const int k_shift = (int)((blockIdx.x + gridDim.x * blockIdx.y) % (unsigned)nk);
+    // Workgroups of different XCDs start their walk over K at different steps
+    // (and wrap around).  With a power-of-two row pitch the rows of one K step
+    // all fall into the same memory channel; if every workgroup asked for the
+    // same step at once, one channel would serve the whole chip.  The
+    // workgroups of ONE XCD (launch number modulo 8) walk in step, so that the
+    // panels they share are fetched into that XCD's L2 once: with a start per
+    // workgroup the fp32 kernel read its operands 20 times over (4.0 GB per
+    // 4096^3 product), with a start per XCD 0.78 GB, and ran 3 % faster.  The
+    // sum over K does not depend on where the walk starts.
+    const int k_shift = (int)((((blockIdx.x + gridDim.x * blockIdx.y) % 8u) * (unsigned)nk) / 8u);
     auto step_of = [&](int kt) {
         const int s = kt + k_shift;
         return s >= nk ? s - nk : s;
@@ -1035,10 +1039,9 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float, 
     if (nk == 0) {
         return;
     }
-    // Concurrent workgroups start their walk over K at different steps, so
-    // that they do not all pull on the same memory channel (see the MFMA
-    // gernel above).
-    const int k_shift = (int)((blockIdx.x + gridDim.x * blockIdx.y) % (unsigned)nk);
+    // The workgroups of one XCD walk over K in step (see the MFMA gernel above);
+    // the eight XCDs start an eighth of K apart.
+    const int k_shift = (int)((((blockIdx.x + gridDim.x * blockIdx.y) % 8u) * (unsigned)nk) / 8u);
     auto step_of = [&](int kt) {
         const int s = kt + k_shift;
         return s >= nk ? s - nk : s;

@@ -126,6 +126,7 @@ struct ScoreTile {
     float sum[2][4];
     float unit;
     int valid_cols;  // columns of the tile that exist (keys)
+    int row0, col0;  // a view of a matrix: where its first element lies
 
     __device__ __forceinline__ void destroy() {
     }
@@ -137,8 +138,11 @@ __device__ __forceinline__ ScoreTile<R, C> allocate_score_tile() {
 }
 
 template<int64_t R, int64_t C>
-__device__ __forceinline__ ScoreTile<R, C> MatrixF32::view_score_tile(int64_t, int64_t) const {
-    return ScoreTile<R, C>();
+__device__ __forceinline__ ScoreTile<R, C> MatrixF32::view_score_tile(int64_t x, int64_t y) const {
+    ScoreTile<R, C> t;
+    t.row0 = (int)x;
+    t.col0 = (int)y;
+    return t;
 }
 
 template<int64_t R, int64_t C>
@@ -400,16 +404,16 @@ __device__ __forceinline__ void close_row_stats(const RowStatsSession &ex, unsig
 
 // out = in * 2^(m - M) / S per row, with (m, s) the tile's own statistics of
 // the row and M, S those of the whole row, combined from the column blocks of
-// the row block through `ex`.  The tile's position comes from the workgroup's
-// place in the grid: column blocks along x, row blocks along y.
+// the row block through `ex`.  The tile's position is that of the view `out`;
+// the grid has one workgroup per column block along x.
 template<int64_t R, int64_t C>
 __device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const RowStatsSession &ex, ScoreTile<R, C> &out) {
     typedef unsigned long long u64;
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
     const int jl = lane % 16;
-    const int bj = (int)blockIdx.x, nbj = (int)gridDim.x;
-    const int64_t row0 = (int64_t)blockIdx.y * R + 32 * w + 4 * (lane / 16);
+    const int bj = out.col0 / (int)C, nbj = (int)gridDim.x;
+    const int64_t row0 = (int64_t)out.row0 + 32 * w + 4 * (lane / 16);
     const u64 tag = ex.tag;
     {
         // lane j < 8 of each DPP row publishes row slot j (tm = j / 4, i = j % 4)

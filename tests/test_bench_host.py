@@ -47,3 +47,12 @@ def test_traffic_is_used_only_for_the_kernel_it_was_measured_on(tmp_path, monkey
 def test_a_missing_traffic_table_means_no_traffic(tmp_path, monkeypatch):
     monkeypatch.setattr(bench, "TRAFFIC_TABLE", str(tmp_path / "absent.md"))
     assert bench.traffic_table() == {}
+
+
+def test_kernel_identity_does_not_depend_on_what_was_generated_before():
+    import gern_amd
+    first = bench.kernel_id(gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY).source)
+    gern_amd.BlurChain("xy", flags=gern_amd.COMPILE_ONLY)  # moves the code generator's counters
+    again = gern_amd.Softmax(4096, flags=gern_amd.COMPILE_ONLY)
+    assert bench.kernel_id(again.source) == first
+    assert bench.kernel_id(gern_amd.Softmax(1000, flags=gern_amd.COMPILE_ONLY).source) != first
