@@ -468,6 +468,45 @@ CASE("matrix.add_rows_and_columns_on_blocks") {
     matrix_add(2);
 }
 
+// Workgroup order in which an XCD takes blocks of 4 x 8 tiles (Runner::Options::xcd_tile_blocks): whatever the
+// grid, every tile is visited exactly once; grids that are not whole blocks keep the plain order.
+CASE("matrix.add_on_blocks_in_xcd_tile_block_order") {
+    auto in = AbstractDataTypePtr(new const annot::MatrixGPU("input_con"));
+    auto out = AbstractDataTypePtr(new const annot::MatrixGPU("output_con"));
+    annot::MatrixAddGPU add;
+    Variable l_x("l_x"), l_y("l_y");
+    Composable program = Global((Tile(out["row"], l_x) || Grid::Unit::BLOCK_X)((Tile(out["col"], l_y) || Grid::Unit::BLOCK_Y)(add(in, out))));
+    if (compileOnly()) {
+        codegen::GeneratorOptions go;
+        go.xcd_tile_blocks = true;
+        codegen::CodeGenerator cg(std::nullopt, go);
+        const std::string text = cg.generate_code(program);
+        REQUIRE(text.find("gern_sb") != std::string::npos);
+        return;
+    }
+    Runner run(program);
+    Runner::Options o;
+    o.filename = "";
+    o.include = " -I " + libraryDir() + " -I " + packageDir();
+    o.xcd_tile_blocks = true;
+    run.compile(o);
+    REQUIRE(run.getSource().find("gern_sb") != std::string::npos);
+    const int64_t shapes[][2] = {{16, 16}, {32, 8}, {8, 32}, {64, 16}, {12, 8}, {4, 8}, {40, 24}};  // tiles along x, along y
+    for (const auto &shape : shapes) {
+        const int64_t rows = 2 * shape[0], cols = 3 * shape[1];
+        impl::MatrixGPU a(rows, cols, cols), b(rows, cols, cols);
+        a.fill(2.0f);
+        b.fill(-5.0f);
+        int64_t lx = 2, ly = 3;
+        REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {l_x.getName(), &lx}, {l_y.getName(), &ly}}));
+        for (float v : b.get()) {
+            REQUIRE_EQ(v, 3.0f);
+        }
+        a.destroy();
+        b.destroy();
+    }
+}
+
 // ---- user-written GEMM schedule staged through LDS -----------------------------------------------
 
 CASE("schedule.gemm_staged_through_lds") {  // gernels/mm/kernel_3.cu:13-118 of the reference
