@@ -46,6 +46,15 @@ int main() {
             expect(gern_qk_softmax_create(d, d == 256 ? 1024 : 4096, compile_only, &p) == 0, "qk create");
             gern_pipeline_destroy(p);
         }
+        expect(gern_blur_chain_create("xyx", 3, 4, 224, 1, compile_only, &p) == 0, "blur, line-aligned store windows");
+        gern_pipeline_destroy(p);
+        expect(gern_qk_softmax_create(128, 4096, compile_only | GERN_PIPELINE_QK_ROW_BLOCKS, &p) == 0, "qk row blocks");
+        gern_pipeline_destroy(p);
+        for (int schedule : {3, 6, 10}) {
+            expect(gern_gemm_schedule_create(schedule, compile_only, &p) == 0, "gemm schedule create");
+            gern_pipeline_destroy(p);
+        }
+        expect(gern_gemm_schedule_create(4, compile_only, &p) != 0 && p == nullptr, "bad schedule");
         // argument errors leave no pipeline behind
         expect(gern_gemm_create(7, compile_only, &p) != 0 && p == nullptr, "bad variant");
         expect(gern_softmax_create(0, 1, compile_only, &p) != 0 && p == nullptr, "bad width");

@@ -2,7 +2,7 @@
 """In-kernel clocks of the matrix-core pipelines, and the machine rates they are
 judged against, on ONE MI355X.
 
-    python -m gern_amd.microbench [gemm_bf16_phases] [gemm_bf16_split] [vendor_gemm] [qk_phases] [mfma_rate] [write_rate]
+    python -m gern_amd.microbench [gemm_bf16_phases] [gemm_bf16_split] [gemm_bf16_operands] [vendor_gemm] [qk_phases] [mfma_rate] [write_rate]
 
 gemm_bf16_phases  the bf16 GEMM 4096^3 kernel as the code generator emits it
                   (same gernel calls, gernels/mm.h), with the 100 MHz
@@ -13,6 +13,9 @@ gemm_bf16_split   the bf16 GEMM 4096^3 and 8192^3 pipeline built three ways and 
                   in turn in one process: as it is, moving the data only (no LDS
                   reads, no MFMAs), and computing only (every stage on what the
                   first two loaded)
+gemm_bf16_operands  the bf16 GEMM 4096^3 pipeline and torch.matmul on random, all-zero
+                  and all-one matrices, in turn: how much of the launch time is the
+                  clock the GPU grants for the data it is given
 vendor_gemm       torch.matmul (the vendor's GEMM library) on the same shapes,
                   bf16 and fp32: what tuned code of the vendor reaches on this GPU
 qk_phases         the same for the QK^T softmax tile kernel (gernels/qk_tiles.h)
@@ -259,6 +262,50 @@ def gemm_bf16_split(gern_amd, torch):
         del pipes
 
 
+def gemm_bf16_operands(gern_amd, torch):
+    from gern_amd import inputs
+    n = 4096
+    A = inputs.to_bf16_bits(inputs.uniform((n, n), 4, -1.0, 1.0))
+    B = inputs.to_bf16_bits(inputs.uniform((n, n), 5, -1.0, 1.0))
+    dA, dB = torch.from_numpy(A.view(np.int16)).cuda(), torch.from_numpy(B.view(np.int16)).cuda()
+    sets = [("uniform [-1, 1)", dA, dB), ("all zero", torch.zeros_like(dA), torch.zeros_like(dB)),
+            ("all one", torch.full_like(dA, 0x3F80), torch.full_like(dB, 0x3F80))]
+    dC = torch.zeros((n, n), device="cuda")
+    g = gern_amd.Gemm("bf16", overwrite=True)
+    out = torch.empty((n, n), device="cuda", dtype=torch.bfloat16)
+
+    def vendor_us(a, b):
+        for _ in range(5):
+            torch.matmul(a, b, out=out)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(60):
+            torch.matmul(a, b, out=out)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 60 * 1e3
+
+    for _ in range(300):
+        g(dA, dB, dC)
+    print("bf16 GEMM 4096^3, the same kernel on different operand VALUES (us per launch, 3 rounds of 60 launches, in turn):")
+    rows = {name: [] for name, _, _ in sets}
+    for _ in range(3):
+        for name, a, b in sets:
+            rows[name].append(_event_us(gern_amd, torch, lambda: g(a, b, dC), 5, 60))
+    for name, t in rows.items():
+        print("  this build, %-16s %s   min %.1f us = %.0f TFLOP/s" % (name + ":", " ".join("%.1f" % x for x in t), min(t), 2.0 * n ** 3 / (min(t) * 1e-6) / 1e12))
+    views = [(name, a.view(torch.bfloat16), b.view(torch.bfloat16)) for name, a, b in sets]
+    for _ in range(200):
+        torch.matmul(views[0][1], views[0][2], out=out)
+    rows = {name: [] for name, _, _ in sets}
+    for _ in range(3):
+        for name, a, b in views:
+            rows[name].append(vendor_us(a, b))
+    for name, t in rows.items():
+        print("  torch.matmul, %-16s %s   min %.1f us = %.0f TFLOP/s" % (name + ":", " ".join("%.1f" % x for x in t), min(t), 2.0 * n ** 3 / (min(t) * 1e-6) / 1e12))
+
+
 def vendor_gemm(gern_amd, torch):
     print("torch.matmul (vendor GEMM library), uniform [-1, 1) operands, us per launch over 5 rounds of 30 launches:")
     for n in (4096, 8192):
@@ -343,7 +390,7 @@ def main():
     import gern_amd
     if gern_amd.device_count() < 1 or not torch.cuda.is_available():
         sys.exit("gern_amd.microbench needs a GPU")
-    probes = {"gemm_bf16_phases": gemm_bf16_phases, "gemm_bf16_split": gemm_bf16_split, "vendor_gemm": vendor_gemm, "qk_phases": qk_phases, "mfma_rate": mfma_rate, "write_rate": write_rate}
+    probes = {"gemm_bf16_phases": gemm_bf16_phases, "gemm_bf16_split": gemm_bf16_split, "gemm_bf16_operands": gemm_bf16_operands, "vendor_gemm": vendor_gemm, "qk_phases": qk_phases, "mfma_rate": mfma_rate, "write_rate": write_rate}
     chosen = sys.argv[1:] or list(probes)
     for name in chosen:
         if name not in probes:
