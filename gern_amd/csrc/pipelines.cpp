@@ -16,6 +16,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <algorithm>
 #include <cstdlib>
 #include <memory>
 #include <sstream>
@@ -87,7 +88,7 @@ int64_t qkWaves(int64_t n) {
 }
 
 // Generates (and, unless compile-only, loads) the program.
-int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_simd = 0) {
+int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_simd = 0, int xcd_band_rows = 0) {
     std::string include = "-I " + packageDir();
     if (const char *extra = std::getenv("GERN_PIPELINE_EXTRA_OPTIONS")) {
         include += std::string(" ") + extra;  // e.g. "-DNAME=value", for experiments
@@ -97,6 +98,7 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
             codegen::GeneratorOptions go;
             go.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
             go.xcd_tile_blocks = (flags & GERN_PIPELINE_XCD_TILE_BLOCKS) != 0;
+            go.xcd_band_rows = xcd_band_rows;
             go.min_waves_per_simd = min_waves_per_simd;
             codegen::CodeGenerator cg(std::nullopt, go);
             p->source = cg.generate_code(program);
@@ -130,6 +132,7 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
         options.include = include;
         options.xcd_remap = !(flags & GERN_PIPELINE_NO_XCD_REMAP);
         options.xcd_tile_blocks = (flags & GERN_PIPELINE_XCD_TILE_BLOCKS) != 0;
+        options.xcd_band_rows = xcd_band_rows;
         options.min_waves_per_simd = min_waves_per_simd;
         p->runner->compile(options);
         p->source = p->runner->getSource();
@@ -208,7 +211,18 @@ int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_row
                 (Tile(output["col"], col_block.bind(tile_cols * waves_per_block)) || Grid::BLOCK_X)(
                     (Tile(output["col"], col.bind(tile_cols)) || Grid::WARP_X)(chain))));
         }
-        int rc = finish(p.get(), program, flags);
+        // XCD order: bands of about 64 output rows (16 rows of 4-row tiles) dealt to the XCDs in turn.  Halo rows
+        // are shared inside a band through that XCD's L2 (one in sixteen tile rows has its lower neighbour on
+        // another XCD), and the eight XCDs stream through one 16 MiB window of an 8192-wide image together
+        // instead of through eight places 32 MiB apart: 8192^2 x,y,x over rotating buffers 92.6 -> 90.3 us,
+        // same buffers 86 -> 78-86 us (measured in one process; bands of 8 rows of tiles 89.8 us, of 32 and
+        // more 94-105 us, one tile row per band 108 us).  GERN_BLUR_BAND_ROWS overrides it for experiments
+        // (0 = one contiguous run of tiles per XCD).
+        int band_rows = (int)std::max<int64_t>(1, 64 / tile_rows);
+        if (const char *v = std::getenv("GERN_BLUR_BAND_ROWS")) {
+            band_rows = std::max(0, std::atoi(v));
+        }
+        int rc = finish(p.get(), program, flags, 0, band_rows);
         if (rc != 0) {
             return rc;
         }

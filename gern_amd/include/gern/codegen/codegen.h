@@ -55,6 +55,8 @@ bool evaluate(const Constraint &c, const EvalEnv &env, bool &value);
 
 struct GeneratorOptions {
     bool xcd_remap = true;
+    // With xcd_remap: rows of tiles per band (0 = one band per XCD); see Runner::Options.
+    int xcd_band_rows = 0;
     // Instead: each XCD takes blocks of 4 x 8 tiles (see Runner::Options).
     bool xcd_tile_blocks = false;
     // Wavefronts per SIMD the kernel must leave room for (second argument of

@@ -42,6 +42,11 @@ public:
         // Spread consecutive workgroups of one XCD over neighbouring tiles
         // (each of the 8 XCDs of an MI355X has its own L2).
         bool xcd_remap = true;
+        // With xcd_remap: 0 gives each XCD ONE contiguous run of tiles (an eighth of
+        // the grid); n > 0 deals bands of n rows of tiles (a row = gridDim.x tiles)
+        // to the XCDs in turn, which keeps the halo sharing inside a band and lets
+        // the eight XCDs stream through one window of memory together.
+        int xcd_band_rows = 0;
         // Instead of that: the 32 workgroups that run on one XCD at a time take a
         // block of 4 x 8 tiles (x by y), for programs whose tiles share operands
         // along both grid axes (a GEMM: 12 operand panels per 32 tiles).  Applies

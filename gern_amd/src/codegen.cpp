@@ -607,6 +607,25 @@ std::string CodeGenerator::generate_code(Composable c) {
                "    const int64_t gern_block_y = gern_by;\n"
                "    const int64_t gern_block_z = blockIdx.z;\n"
                "    (void)gern_block_x; (void)gern_block_y; (void)gern_block_z;\n";
+    } else if (device && em.uses_block_units && options.xcd_remap && options.xcd_band_rows > 0) {
+        // The same idea with shorter runs: XCD x takes bands x, x + 8, x + 16, ... of `xcd_band_rows` rows of
+        // tiles each (a row = gridDim.x tiles), so that at any time the eight XCDs work side by side in one
+        // window of the data instead of in eight places an eighth of the data apart.  Launch numbers past the
+        // last whole group of eight bands keep their tiles.
+        out << "    const unsigned gern_nbx = gridDim.x, gern_nby = gridDim.y;\n"
+               "    unsigned gern_wg = blockIdx.x + gern_nbx * (blockIdx.y + gern_nby * blockIdx.z);\n"
+               "    {\n"
+               "        const unsigned gern_band = " << options.xcd_band_rows << "u * gern_nbx;\n"
+               "        const unsigned gern_whole = ((gern_nbx * gern_nby * gridDim.z) / (8u * gern_band)) * (8u * gern_band);\n"
+               "        if (gern_wg < gern_whole) {\n"
+               "            const unsigned gern_l = gern_wg / 8u;\n"
+               "            gern_wg = ((gern_l / gern_band) * 8u + gern_wg % 8u) * gern_band + gern_l % gern_band;\n"
+               "        }\n"
+               "    }\n"
+               "    const int64_t gern_block_x = gern_wg % gern_nbx;\n"
+               "    const int64_t gern_block_y = (gern_wg / gern_nbx) % gern_nby;\n"
+               "    const int64_t gern_block_z = gern_wg / (gern_nbx * gern_nby);\n"
+               "    (void)gern_block_x; (void)gern_block_y; (void)gern_block_z;\n";
     } else if (device && em.uses_block_units && options.xcd_remap) {
         // Workgroups are handed to the 8 XCDs round-robin in launch order.
         // Renumbering them so that each XCD walks a contiguous run of tiles

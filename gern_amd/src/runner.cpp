@@ -84,6 +84,7 @@ void Runner::compile(Options config) {
     codegen::GeneratorOptions gen_options;
     gen_options.xcd_remap = config.xcd_remap;
     gen_options.xcd_tile_blocks = config.xcd_tile_blocks;
+    gen_options.xcd_band_rows = config.xcd_band_rows;
     gen_options.min_waves_per_simd = config.min_waves_per_simd;
     codegen::CodeGenerator cg(ordered_parameters, gen_options);
     source = cg.generate_code(c);

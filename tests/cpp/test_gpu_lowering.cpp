@@ -507,6 +507,48 @@ CASE("matrix.add_on_blocks_in_xcd_tile_block_order") {
     }
 }
 
+// Bands of rows of tiles dealt to the XCDs in turn (Runner::Options::xcd_band_rows): every tile is visited
+// exactly once, also when the grid is not a whole number of groups of eight bands.
+CASE("matrix.add_on_blocks_in_xcd_band_order") {
+    auto in = AbstractDataTypePtr(new const annot::MatrixGPU("input_con"));
+    auto out = AbstractDataTypePtr(new const annot::MatrixGPU("output_con"));
+    annot::MatrixAddGPU add;
+    Variable l_x("l_x"), l_y("l_y");
+    // columns on BLOCK_X, rows on BLOCK_Y: a row of tiles is gridDim.x tiles, as in the blur
+    Composable program = Global((Tile(out["row"], l_x) || Grid::Unit::BLOCK_Y)((Tile(out["col"], l_y) || Grid::Unit::BLOCK_X)(add(in, out))));
+    for (int band_rows : {1, 3, 16}) {
+        if (compileOnly()) {
+            codegen::GeneratorOptions go;
+            go.xcd_band_rows = band_rows;
+            codegen::CodeGenerator cg(std::nullopt, go);
+            REQUIRE(cg.generate_code(program).find("gern_band") != std::string::npos);
+            continue;
+        }
+        Runner run(program);
+        Runner::Options o;
+        o.filename = "";
+        o.include = " -I " + libraryDir() + " -I " + packageDir();
+        o.xcd_band_rows = band_rows;
+        run.compile(o);
+        REQUIRE(run.getSource().find("gern_band") != std::string::npos);
+        const int64_t shapes[][2] = {{128, 5}, {24, 7}, {49, 3}, {8, 1}, {7, 2}, {300, 4}};  // rows of tiles, tiles per row
+        for (const auto &shape : shapes) {
+            const int64_t rows = 2 * shape[0], cols = 3 * shape[1];
+            impl::MatrixGPU a(rows, cols, cols), b(rows, cols, cols);
+            a.fill(2.0f);
+            b.fill(-5.0f);
+            int64_t lx = 2, ly = 3;
+            REQUIRE_NOTHROW(run.evaluate({{in.getName(), &a}, {out.getName(), &b}, {l_x.getName(), &lx}, {l_y.getName(), &ly}}));
+            for (float v : b.get()) {
+                REQUIRE_EQ(v, 3.0f);
+            }
+            a.destroy();
+            b.destroy();
+        }
+        run.release();
+    }
+}
+
 // ---- user-written GEMM schedule staged through LDS -----------------------------------------------
 
 CASE("schedule.gemm_staged_through_lds") {  // gernels/mm/kernel_3.cu:13-118 of the reference
