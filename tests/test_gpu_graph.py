@@ -17,6 +17,10 @@ def test_pipelines_replay_from_a_hip_graph(oracle):
     blur = gpu.BlurChain("xyx", tile_rows=6)
     sm = gpu.Softmax(1024)
     gemm = gpu.Gemm("bf16", overwrite=True)
+    # the 256 x 256 tile kernel: two row blocks x two column blocks exchange row statistics through device
+    # memory; its launch number lives there too, so a replay is a launch like any other
+    qk = gpu.QKSoftmax(128, 512)
+    m_q, n_k, d_h = 300, 512, 128
     shape_img, shape_x, n = (200, 520), (48, 1024), 256
     d_img = torch.zeros(shape_img, device="cuda")
     d_blur = torch.zeros(blur.out_shape(*shape_img), device="cuda")
@@ -25,6 +29,10 @@ def test_pipelines_replay_from_a_hip_graph(oracle):
     d_a = torch.zeros((n, n), dtype=torch.int16, device="cuda")
     d_b = torch.zeros((n, n), dtype=torch.int16, device="cuda")
     d_c = torch.zeros((n, n), device="cuda")
+    d_q = torch.zeros((m_q, d_h), dtype=torch.int16, device="cuda")
+    d_k = torch.zeros((n_k, d_h), dtype=torch.int16, device="cuda")
+    d_s = torch.zeros((m_q, n_k), device="cuda")
+    scale = np.float32(1.0 / np.sqrt(d_h))
 
     side = torch.cuda.Stream()  # default priority
 
@@ -33,6 +41,7 @@ def test_pipelines_replay_from_a_hip_graph(oracle):
         blur(d_img, d_blur, stream=h)
         sm(d_x, d_y, stream=h)
         gemm(d_a, d_b, d_c, stream=h)
+        qk(d_q, d_k, d_s, scale, stream=h)
 
     # everything that loads code or queries the device happens before capture
     with torch.cuda.stream(side):
@@ -55,7 +64,11 @@ def test_pipelines_replay_from_a_hip_graph(oracle):
         d_x.copy_(torch.from_numpy(x))
         d_a.copy_(torch.from_numpy(ab.view(np.int16)))
         d_b.copy_(torch.from_numpy(bb.view(np.int16)))
-        for out in (d_blur, d_y, d_c):
+        qb, _ = oracle.to_bf16(oracle.normal((m_q, d_h), 500 + rep))
+        kb, _ = oracle.to_bf16(oracle.normal((n_k, d_h), 600 + rep))
+        d_q.copy_(torch.from_numpy(qb.view(np.int16)))
+        d_k.copy_(torch.from_numpy(kb.view(np.int16)))
+        for out in (d_blur, d_y, d_c, d_s):
             out.fill_(float("nan"))
         torch.cuda.synchronize()
         graph.replay()
@@ -64,3 +77,7 @@ def test_pipelines_replay_from_a_hip_graph(oracle):
         want = oracle.softmax_rows(x)
         assert np.max(np.abs(d_y.cpu().numpy() - want) / want) < 1e-5, rep
         assert np.array_equal(d_c.cpu().numpy(), ai @ bi), rep
+        want = oracle.qk_softmax(qb, kb, scale)
+        got = d_s.cpu().numpy()
+        assert np.all(np.isfinite(got)), rep
+        assert np.max(np.abs(got - want) / want) < 1e-2, rep
