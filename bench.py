@@ -240,6 +240,24 @@ def cpu_blur(img_np, pattern, tile_rows, tile_cols, budget_s, what_size):
     }
 
 
+def cpu_time(run, budget_s, nbytes=None, flop=None, what=""):
+    """Median of up to five runs (after one warm-up) of a CPU pipeline on ONE host core."""
+    run()
+    times = []
+    budget = time.perf_counter() + budget_s
+    while len(times) < 5 and (len(times) < 1 or time.perf_counter() < budget):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    out = {"cores": 1, "host_cores": os.cpu_count(), "seconds": med, "sample": "%s; median of %d runs after one warm-up" % (what, len(times))}
+    if nbytes is not None:
+        out.update({"value": nbytes / med / 1e9, "unit": "GB/s"})
+    if flop is not None:
+        out.update({"value": flop / med / 1e9, "unit": "GFLOP/s"})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -381,6 +399,20 @@ def main():
             roof = roofline("softmax_8192x4096", table, "hbm", 2 * x.nbytes, t, sm)
             workloads["softmax_8192x4096"] = {"GB/s": roof["achieved"], "ms": t["ms"], "frac_hbm": roof["frac"], "roofline": roof}
             log("softmax 8192x4096: %.1f us  %.0f GB/s (%.1f%%)" % (t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"]))
+        if not args.no_cpu and not args.rotating_only:
+            from oracle import oracle as o
+            from oracle import ref
+            sample = x[:1024]  # 1024 of the 8192 rows: a bounded sample of the same workload
+            if ref.available():
+                cpu = cpu_time(lambda: ref.softmax_rows(sample), 5.0, nbytes=2 * sample.nbytes,
+                               what="1024 rows of the 8192x4096 softmax, reference library CPU lowering of the fused five-gernel pipeline, g++ -O2")
+                cpu["kind"] = "reference"
+            else:
+                cpu = cpu_time(lambda: o.softmax_rows(sample), 5.0, nbytes=2 * sample.nbytes,
+                               what="1024 rows of the 8192x4096 softmax, CPU oracle, gcc -O2")
+                cpu["kind"] = "port"
+            workloads["softmax_8192x4096_cpu"] = cpu
+            log("softmax on the CPU (1024 rows): %.2f GB/s on 1 core (%s)" % (cpu["value"], cpu["kind"]))
         if not args.no_rotating:
             ring = [(d_x, d_y)] + [(d_x.clone(), torch.zeros_like(d_y)) for _ in range(5)]
             tr = measure(rotating(ring, lambda a, b: sm(a, b)), args.warmup, steps2, torch, gern_amd)
@@ -410,6 +442,19 @@ def main():
         workloads["gemm_%s_4096" % variant] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
                                                "peak_TFLOP/s": roof["peak"], "roofline": roof}
         log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], roof["peak"]))
+        if variant == "f32" and not args.no_cpu:
+            from oracle import oracle as o
+            from oracle import ref
+            As, Bs = A[:512, :512].copy(), B[:512, :512].copy()  # a 512^3 corner of the product: 1/512 of the flops
+            if ref.available():
+                cpu = cpu_time(lambda: ref.gemm(As, Bs, 64, 64, 64), 8.0, flop=2.0 * 512 ** 3,
+                               what="512^3 corner of the 4096^3 fp32 product, reference library CPU lowering of Tile(64)(Tile(64)(Reduce(64)(matrix_multiply))), g++ -O2")
+                cpu["kind"] = "reference"
+            else:
+                cpu = cpu_time(lambda: o.gemm_f32(As, Bs), 8.0, flop=2.0 * 512 ** 3, what="512^3 corner of the 4096^3 fp32 product, CPU oracle, gcc -O2")
+                cpu["kind"] = "port"
+            workloads["gemm_f32_512_cpu"] = cpu
+            log("gemm f32 512^3 on the CPU: %.2f GFLOP/s on 1 core (%s)" % (cpu["value"], cpu["kind"]))
         if variant == "f32":
             # the same product on the kernel that takes every shape (vector-ALU FMAs)
             g = gern_amd.Gemm(variant, overwrite=True, general_only=True)
