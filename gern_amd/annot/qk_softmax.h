@@ -193,34 +193,12 @@ public:
     }
 };
 
-// out = 2^(in - rowmax) with the row statistics of the tile kept beside it.
-class ExpRows : public ExpMatrix {
+// out = the softmax over WHOLE rows of the matrix that `input` is a tile of
+// scaled products of; the tiles of a row block exchange their row statistics
+// through `exchange` (gernels::softmax_rows_across_tiles).
+class SoftmaxAcrossTiles : public AbstractFunction {
 public:
-    using ExpMatrix::ExpMatrix;
-    FunctionSignature getFunction() override {
-        FunctionSignature f = ExpMatrix::getFunction();
-        f.name = "gernels::exp_rows";
-        return f;
-    }
-    Annotation getAnnotation() override {
-        Variable x("x"), y("y");
-        Variable l_x("l_x", Datatype::Int64, true), l_y("l_y", Datatype::Int64, true);
-        return Tileable(x = Expr(0), ADTMember(output, "row", false), l_x,
-                        Tileable(y = Expr(0), ADTMember(output, "col", false), l_y,
-                                 Produces::Subset(output, {x, y, l_x, l_y}),
-                                 Consumes::Subset(input, {x, y, l_x, l_y})))
-            .occupies({Grid::Unit::THREAD_X});
-    }
-    std::vector<std::string> getHeader() override {
-        return {"gernels/qk_tiles.h"};
-    }
-};
-
-// out = in scaled per row to the softmax of the WHOLE row; the tiles of a row
-// block exchange their statistics through `exchange`.
-class NormaliseRows : public AbstractFunction {
-public:
-    NormaliseRows(AbstractDataTypePtr input, AbstractDataTypePtr exchange, AbstractDataTypePtr output)
+    SoftmaxAcrossTiles(AbstractDataTypePtr input, AbstractDataTypePtr exchange, AbstractDataTypePtr output)
         : input(input), exchange(exchange), output(output) {
     }
     Annotation getAnnotation() override {
@@ -237,7 +215,7 @@ public:
     }
     FunctionSignature getFunction() override {
         FunctionSignature f;
-        f.name = "gernels::normalise_rows";
+        f.name = "gernels::softmax_rows_across_tiles";
         f.args = {Parameter(input), Parameter(exchange), Parameter(output)};
         return f;
     }

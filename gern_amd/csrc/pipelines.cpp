@@ -543,13 +543,11 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
             using Tile256 = annot::ScoreTileF32;
             auto S = AbstractDataTypePtr(new const Tile256("S", Tile256::OUTPUT));
             auto logits = AbstractDataTypePtr(new const Tile256("logits", Tile256::TEMP));
-            auto expd = AbstractDataTypePtr(new const Tile256("expd", Tile256::TEMP));
             auto exchange = AbstractDataTypePtr(new const annot::RowStatsExchange("exchange"));
             annot::QKScaled qk{Q, K, logits};
-            annot::ExpRows ex{logits, expd};
-            annot::NormaliseRows norm{expd, exchange, S};
+            annot::SoftmaxAcrossTiles softmax{logits, exchange, S};
             program = Global((Tile(S["row"], rows.bind(256)) || Grid::BLOCK_Y)((Tile(S["col"], keys.bind(256)) || Grid::BLOCK_X)(
-                                 qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), ex(logits, expd), norm(expd, exchange, S))),
+                                 qk[{{"d", d.bind(head_dim)}}](Q, K, logits, scale), softmax(logits, exchange, S))),
                              {{Grid::BLOCK_DIM_X, threads.bind(512)}});
         } else {
             auto S = AbstractDataTypePtr(new const annot::RowBlockF32("S", annot::RowBlockF32::OUTPUT));

@@ -8,18 +8,25 @@
 // the workgroups of a row block combine their row statistics through global
 // memory while the tiles wait in registers:
 //
-//   qk_scaled       MFMA: the tile's logits, kept as raw accumulators plus the
-//                   factor that turns them into log2 units
-//   exp_rows        per row of the tile: maximum m, e = 2^(x - m), sum s of e
-//   normalise_rows  publishes (m, s) per row, waits for the same from the
-//                   other tiles of the row block, and scales e by
-//                   2^(m - M) / S with M, S the statistics of the whole row
+//   qk_scaled                    MFMA: the tile's logits, kept as raw accumulators plus
+//                                the factor that turns them into log2 units
+//   softmax_rows_across_tiles    per row of the tile: maximum m, e = 2^(x - m), sum s
+//                                of e; publishes (m, s), waits for the same from the
+//                                other tiles of the row block, scales e by
+//                                2^(m - M) / S with M, S the statistics of the whole
+//                                row, and stores
 //
 // so a softmax over tiled rows is the five stages of the reference's softmax
 // gernels (apps/common/impl/impl.h:7-188: max, subtract, exp, sum, divide) with
 // the two reductions finished across workgroups, as the reference's
 // grid_reduce_total finishes a sum across blocks with a device-scope atomic
-// (gernels/cccl/wrappers/reduce_wrappers.cuh:42-61).
+// (gernels/cccl/wrappers/reduce_wrappers.cuh:42-61).  The five stages are ONE
+// gernel here because they are pipelined over the two 16-row halves of a
+// wavefront's rows: the statistics of the first half are on their way to the
+// other workgroups while the exponentials of the second are computed, and the
+// first half is being stored while the second waits for its statistics (as
+// three gernels with one exchange for all rows: 25.1 us at 4096 x 4096 x 128;
+// this way 22.2 us, measured in one process).
 //
 // Eight wavefronts; wavefront w owns rows [32 w, 32 w + 32) of the tile and all
 // 256 columns, as 2 x 16 v_mfma_f32_16x16x32_bf16 tiles.  MFMA column j of
@@ -27,7 +34,7 @@
 // consecutive columns of S per group g and stores them with one 16-byte store.
 //
 // The exchange.  An entry is one 64-bit word per (row, column block): s in the
-// upper half, below it m as a sixteen-bit integer (exp_rows shifts a row by
+// upper half, below it m as a sixteen-bit integer (a row is shifted by
 // the floor of its largest logit in log2 units: any shift near the maximum
 // serves, and a whole number makes 2^(m - M) an exact power of two), and a
 // sixteen-bit tag.  The tag is the launch's number, which is kept in device
@@ -103,9 +110,9 @@ struct RowStatsExchange {
 
 namespace detail {
 // Wavefronts of the workgroup that are done with the exchange.  qk_scaled clears
-// it ahead of its first barrier and normalise_rows counts in it, so that
-// normalise_rows needs no barrier of its own: the wavefronts of a workgroup
-// finish exp_rows up to a microsecond or two apart (a SIMD serves its older
+// it ahead of its first barrier and softmax_rows_across_tiles counts in it, so
+// that the exchange needs no barrier of its own: the wavefronts of a workgroup
+// finish their exponentials up to a microsecond or two apart (a SIMD serves its older
 // wavefront first), and a wavefront exchanges only with its namesakes in the
 // other tiles of the row block, so the early ones are storing their rows while
 // the late ones still compute.
@@ -114,7 +121,7 @@ __shared__ unsigned int row_stats_waves_done;
 
 // A 256 x 256 tile of scores spread over eight wavefronts: acc[tm][4 g + t][i]
 // is row 32 w + 16 tm + 4 (lane / 16) + i, column 64 g + 4 (lane % 16) + t,
-// in units of `unit` (value = acc * unit) until exp_rows, plain afterwards.
+// in units of `unit` (value = acc * unit) as qk_scaled leaves it, plain afterwards.
 // shift / sum: the statistics of the lane's eight rows over the tile's columns.
 template<int64_t R, int64_t C>
 struct ScoreTile {
@@ -126,7 +133,12 @@ struct ScoreTile {
     float sum[2][4];
     float unit;
     int valid_cols;  // columns of the tile that exist (keys)
-    int row0, col0;  // a view of a matrix: where its first element lies
+    // A view of a matrix (view_score_tile): the matrix and where the tile's first
+    // element lies in it.  A gernel may write its rows through the view as they
+    // become final; `stored` then tells store_score_tile that nothing is left.
+    MatrixF32 home;
+    int row0, col0;
+    bool stored;
 
     __device__ __forceinline__ void destroy() {
     }
@@ -134,45 +146,65 @@ struct ScoreTile {
 
 template<int64_t R, int64_t C>
 __device__ __forceinline__ ScoreTile<R, C> allocate_score_tile() {
-    return ScoreTile<R, C>();
+    ScoreTile<R, C> t;
+    t.home = MatrixF32{nullptr, 0, 0, 0};
+    t.row0 = t.col0 = 0;
+    t.stored = false;
+    return t;
 }
 
 template<int64_t R, int64_t C>
 __device__ __forceinline__ ScoreTile<R, C> MatrixF32::view_score_tile(int64_t x, int64_t y) const {
     ScoreTile<R, C> t;
+    t.home = *this;
     t.row0 = (int)x;
     t.col0 = (int)y;
+    t.stored = false;
     return t;
 }
 
+namespace detail {
+
+// Row 16 tm + i of each lane's rows (32 w + 4 (lane / 16) + that), every value
+// times f, 16 bytes per lane and store.
 template<int64_t R, int64_t C>
-__device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y, const ScoreTile<R, C> &t) const {
+__device__ __forceinline__ void store_score_row(const MatrixF32 &m, int64_t x, int64_t y, const ScoreTile<R, C> &t, int tm, int i, float f) {
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
     const int jl = lane % 16;
+    const int64_t rr = x + 32 * w + 16 * tm + 4 * (lane / 16) + i;
+    if (rr >= m.row) {
+        return;
+    }
+    float *p = m.data + rr * m.lda;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const int64_t cc = y + 64 * g + 4 * jl;
+        const float4 val = make_float4(t.acc[tm][4 * g + 0][i] * f, t.acc[tm][4 * g + 1][i] * f, t.acc[tm][4 * g + 2][i] * f,
+                                       t.acc[tm][4 * g + 3][i] * f);
+        if (cc + 3 < m.col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
+            store_streaming(p + cc, val);
+        } else {
+            if (cc + 0 < m.col) p[cc + 0] = val.x;
+            if (cc + 1 < m.col) p[cc + 1] = val.y;
+            if (cc + 2 < m.col) p[cc + 2] = val.z;
+            if (cc + 3 < m.col) p[cc + 3] = val.w;
+        }
+    }
+}
+
+}  // namespace detail
+
+template<int64_t R, int64_t C>
+__device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y, const ScoreTile<R, C> &t) const {
+    if (t.stored) {  // its rows went out through the view
+        return;
+    }
 #pragma unroll
     for (int tm = 0; tm < 2; tm++) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int64_t rr = x + 32 * w + 16 * tm + 4 * (lane / 16) + i;
-            if (rr >= row) {
-                continue;
-            }
-            float *p = data + rr * lda;
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int64_t cc = y + 64 * g + 4 * jl;
-                const float4 val = make_float4(t.acc[tm][4 * g + 0][i], t.acc[tm][4 * g + 1][i], t.acc[tm][4 * g + 2][i],
-                                               t.acc[tm][4 * g + 3][i]);
-                if (cc + 3 < col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
-                    store_streaming(p + cc, val);
-                } else {
-                    if (cc + 0 < col) p[cc + 0] = val.x;
-                    if (cc + 1 < col) p[cc + 1] = val.y;
-                    if (cc + 2 < col) p[cc + 2] = val.z;
-                    if (cc + 3 < col) p[cc + 3] = val.w;
-                }
-            }
+            detail::store_score_row(*this, x, y, t, tm, i, 1.0f);
         }
     }
 }
@@ -188,7 +220,7 @@ __device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y
 // MFMA tile 4 g + t are then sixteen consecutive LDS rows, like the rows of Q.
 // Rows of Q and keys past the end of the matrices are read from the last
 // valid one (rows past the end are never stored, keys past the end are left
-// out of the statistics by exp_rows).
+// out of the statistics by softmax_rows_across_tiles).
 template<int64_t R, int64_t C, int64_t D>
 __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false> &Q, const GlobalView<C, D, uint16_t, false> &K,
                                           ScoreTile<R, C> &S, float scale) {
@@ -293,73 +325,6 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
     }
 }
 
-// out = 2^(in - m) per row of the tile, m the row's maximum over the tile's
-// valid columns; out.shift = m, out.sum = the sum of the row's 2^(in - m).
-template<int64_t R, int64_t C>
-__device__ __forceinline__ void exp_rows(const ScoreTile<R, C> &in, ScoreTile<R, C> &out) {
-    const int jl = lane_id() % 16;
-    const float unit = in.unit;
-    const bool partial = in.valid_cols < (int)C;  // workgroup-uniform: the last column block only
-    const bool flip = unit < 0.f;                 // a negative scale turns the largest product into the smallest logit
-    out.unit = 1.0f;
-    out.valid_cols = in.valid_cols;
-#pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float x[16];
-#pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                x[tn] = in.acc[tm][tn][i];
-            }
-            if (flip) {
-#pragma unroll
-                for (int tn = 0; tn < 16; tn++) {
-                    x[tn] = -x[tn];
-                }
-            }
-            if (partial) {
-#pragma unroll
-                for (int tn = 0; tn < 16; tn++) {
-                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
-                    x[tn] = key < in.valid_cols ? x[tn] : -__builtin_huge_valf();
-                }
-            }
-            float m = x[0];
-#pragma unroll
-            for (int tn = 1; tn < 16; tn++) {
-                m = __builtin_fmaxf(m, x[tn]);
-            }
-            m = __builtin_fmaxf(m, dpp_move<0xB1>(m));   // the sixteen lanes of a DPP row share the tile's rows
-            m = __builtin_fmaxf(m, dpp_move<0x4E>(m));
-            m = __builtin_fmaxf(m, dpp_move<0x141>(m));
-            m = __builtin_fmaxf(m, dpp_move<0x140>(m));
-            const float a = flip ? -unit : unit;
-            // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
-            // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
-            const float shift = __builtin_fminf(__builtin_fmaxf(__builtin_floorf(m * a), -32768.0f), 32767.0f);
-            float s = 0.f;
-#pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                // a masked column is -inf: 2^-inf = 0 unless a == 0 (0 * inf), which the test below catches
-                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(x[tn], a, -shift));
-                if (partial) {
-                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
-                    e = key < in.valid_cols ? e : 0.f;
-                }
-                out.acc[tm][tn][i] = e;
-                s += e;
-            }
-            s += dpp_move<0xB1>(s);
-            s += dpp_move<0x4E>(s);
-            s += dpp_move<0x141>(s);
-            s += dpp_move<0x140>(s);
-            out.shift[tm][i] = shift;
-            out.sum[tm][i] = s;
-        }
-    }
-}
-
 namespace detail {
 
 // The last workgroup of a launch advances the launch number and clears the
@@ -402,105 +367,184 @@ __device__ __forceinline__ void close_row_stats(const RowStatsSession &ex, unsig
 
 }  // namespace detail
 
-// out = in * 2^(m - M) / S per row, with (m, s) the tile's own statistics of
-// the row and M, S those of the whole row, combined from the column blocks of
-// the row block through `ex`.  The tile's position is that of the view `out`;
-// the grid has one workgroup per column block along x.
+// out = softmax over the WHOLE rows of S that the tile `in` of scaled products
+// (value = acc * in.unit, in log2 units) is a 256-column piece of; `out` is a
+// view of S and its rows are stored through it.  Per 16-row half of a
+// wavefront's rows, in this order:
+//
+//   half 0: m = floor(max), e = 2^(x - m), s = sum e; publish (m, s) per row
+//   half 1: the same
+//   half 0: wait for the sixteen column blocks' (m, s) of its rows, combine to
+//           (M, S), store e * 2^(m - M) / S
+//   half 1: the same
+//
+// so the entries of half 0 travel while half 1 is computed, and half 0 is
+// stored while half 1 waits.  An entry is published by lanes j < 4 of each
+// 16-lane row (row slot i = j of the half).
 template<int64_t R, int64_t C>
-__device__ __forceinline__ void normalise_rows(const ScoreTile<R, C> &in, const RowStatsSession &ex, ScoreTile<R, C> &out) {
+__device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> &in, const RowStatsSession &ex, ScoreTile<R, C> &out) {
     typedef unsigned long long u64;
+    // Rows per lane and pipeline step (slot r = 4 tm + i is row 16 tm + i of the lane's eight rows).  Measured
+    // at 4096 x 4096 x 128 in one process: 8 (one exchange for all rows) 24.3 us, 4 (the two halves) 21.7 us,
+    // 1 (row by row) 23.6 us.
+#ifndef GERN_QK_GROUP
+#define GERN_QK_GROUP 4
+#endif
+    constexpr int G = GERN_QK_GROUP;
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8, "group size");
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
     const int jl = lane % 16;
-    const int bj = out.col0 / (int)C, nbj = (int)gridDim.x;
+    const float unit = in.unit;
+    const bool partial = in.valid_cols < (int)C;  // workgroup-uniform: the last column block only
+    const bool flip = unit < 0.f;                 // a negative scale turns the largest product into the smallest logit
+    const int bj = out.col0 / (int)C, nbj = (int)gridDim.x;  // one workgroup per column block along x
     const int64_t row0 = (int64_t)out.row0 + 32 * w + 4 * (lane / 16);
     const u64 tag = ex.tag;
-    {
-        // lane j < 8 of each DPP row publishes row slot j (tm = j / 4, i = j % 4)
-        float m = in.shift[0][0], s = in.sum[0][0];
-#pragma unroll
-        for (int q = 1; q < 8; q++) {
-            m = jl == q ? in.shift[q / 4][q % 4] : m;
-            s = jl == q ? in.sum[q / 4][q % 4] : s;
-        }
-        if (jl < 8) {
-            u64 *e = ex.entries + ((row0 + 16 * (jl / 4) + (jl % 4)) * ex.pitch + bj);
-            const u64 word = ((u64)(unsigned int)as_int(s) << 32) | ((u64)((unsigned int)(int)m & 0xFFFFu) << 16) | tag;
-            __hip_atomic_store(e, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    // Lane j collects column block j (j + 16, ...) for its eight rows.
-    float big_m[2][4], big_s[2][4];
-#pragma unroll
-    for (int q = 0; q < 8; q++) {
-        big_m[q / 4][q % 4] = -__builtin_huge_valf();
-        big_s[q / 4][q % 4] = 0.f;
-    }
-    bool failed = false;
-    for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
-        const int b = b0 + jl;
-        u64 got[8];
-        int spins = 0;
-        for (;;) {
-            bool mine = true;
-            if (b < nbj) {
-#pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    const u64 *e = ex.entries + ((row0 + 16 * (q / 4) + (q % 4)) * ex.pitch + b);
-                    got[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-                for (int q = 0; q < 8; q++) {
-                    mine = mine && (got[q] & 0xFFFFull) == tag;
-                }
-            }
-            if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
-                break;
-            }
-            if (++spins > ex.spin_limit) {  // wave-uniform
-                failed = true;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(GERN_QK_SLEEP);
-        }
-        if (b < nbj) {
-#pragma unroll
-            for (int q = 0; q < 8; q++) {
-                const float m = (float)(short)(unsigned short)((got[q] >> 16) & 0xFFFFull), s = as_float((int)(unsigned int)(got[q] >> 32));
-                const float top = __builtin_fmaxf(big_m[q / 4][q % 4], m);
-                big_s[q / 4][q % 4] = big_s[q / 4][q % 4] * __builtin_amdgcn_exp2f(big_m[q / 4][q % 4] - top) +
-                                      s * __builtin_amdgcn_exp2f(m - top);
-                big_m[q / 4][q % 4] = top;
-            }
-        }
-    }
-    detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
     out.unit = 1.0f;
     out.valid_cols = in.valid_cols;
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
+    for (int grp = 0; grp < 8 / G; grp++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float m = big_m[tm][i];
+        for (int r = grp * G; r < grp * G + G; r++) {
+            const int tm = r / 4, i = r % 4;
+            float x[16];
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                x[tn] = in.acc[tm][tn][i];
+            }
+            if (flip) {
+#pragma unroll
+                for (int tn = 0; tn < 16; tn++) {
+                    x[tn] = -x[tn];
+                }
+            }
+            if (partial) {
+#pragma unroll
+                for (int tn = 0; tn < 16; tn++) {
+                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
+                    x[tn] = key < in.valid_cols ? x[tn] : -__builtin_huge_valf();
+                }
+            }
+            float m = x[0];
+#pragma unroll
+            for (int tn = 1; tn < 16; tn++) {
+                m = __builtin_fmaxf(m, x[tn]);
+            }
+            m = __builtin_fmaxf(m, dpp_move<0xB1>(m));
+            m = __builtin_fmaxf(m, dpp_move<0x4E>(m));
+            m = __builtin_fmaxf(m, dpp_move<0x141>(m));
+            m = __builtin_fmaxf(m, dpp_move<0x140>(m));
+            const float a = flip ? -unit : unit;
+            // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
+            // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
+            const float shift = __builtin_fminf(__builtin_fmaxf(__builtin_floorf(m * a), -32768.0f), 32767.0f);
+            float s = 0.f;
+#pragma unroll
+            for (int tn = 0; tn < 16; tn++) {
+                // a masked column is -inf: 2^-inf = 0 unless a == 0 (0 * inf), which the test below catches
+                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(x[tn], a, -shift));
+                if (partial) {
+                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
+                    e = key < in.valid_cols ? e : 0.f;
+                }
+                out.acc[tm][tn][i] = e;
+                s += e;
+            }
+            s += dpp_move<0xB1>(s);
+            s += dpp_move<0x4E>(s);
+            s += dpp_move<0x141>(s);
+            s += dpp_move<0x140>(s);
+            out.shift[tm][i] = shift;
+            out.sum[tm][i] = s;
+        }
+        {
+            // lane j < G of each 16-lane row publishes slot grp * G + j
+            float m = out.shift[(grp * G) / 4][(grp * G) % 4], s = out.sum[(grp * G) / 4][(grp * G) % 4];
+#pragma unroll
+            for (int q = 1; q < G; q++) {
+                m = jl == q ? out.shift[(grp * G + q) / 4][(grp * G + q) % 4] : m;
+                s = jl == q ? out.sum[(grp * G + q) / 4][(grp * G + q) % 4] : s;
+            }
+            if (jl < G) {
+                const int r = grp * G + jl;
+                u64 *e = ex.entries + ((row0 + 16 * (r / 4) + (r % 4)) * ex.pitch + bj);
+                const u64 word = ((u64)(unsigned int)as_int(s) << 32) | ((u64)((unsigned int)(int)m & 0xFFFFu) << 16) | tag;
+                __hip_atomic_store(e, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+#pragma unroll
+    for (int grp = 0; grp < 8 / G; grp++) {
+        // Lane j collects column block j (j + 16, ...) for the G rows it holds of this group.
+        float big_m[G], big_s[G];
+#pragma unroll
+        for (int q = 0; q < G; q++) {
+            big_m[q] = -__builtin_huge_valf();
+            big_s[q] = 0.f;
+        }
+        bool failed = false;
+        for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
+            const int b = b0 + jl;
+            u64 got[G];
+            int spins = 0;
+            for (;;) {
+                bool mine = true;
+                if (b < nbj) {
+#pragma unroll
+                    for (int q = 0; q < G; q++) {
+                        const int r = grp * G + q;
+                        const u64 *e = ex.entries + ((row0 + 16 * (r / 4) + (r % 4)) * ex.pitch + b);
+                        got[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int q = 0; q < G; q++) {
+                        mine = mine && (got[q] & 0xFFFFull) == tag;
+                    }
+                }
+                if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
+                    break;
+                }
+                if (++spins > ex.spin_limit) {  // wave-uniform
+                    failed = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(GERN_QK_SLEEP);
+            }
+            if (b < nbj) {
+#pragma unroll
+                for (int q = 0; q < G; q++) {
+                    const float m = (float)(short)(unsigned short)((got[q] >> 16) & 0xFFFFull), s = as_float((int)(unsigned int)(got[q] >> 32));
+                    const float top = __builtin_fmaxf(big_m[q], m);
+                    big_s[q] = big_s[q] * __builtin_amdgcn_exp2f(big_m[q] - top) + s * __builtin_amdgcn_exp2f(m - top);
+                    big_m[q] = top;
+                }
+            }
+        }
+        if (grp == 8 / G - 1) {
+            detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
+        }
+#pragma unroll
+        for (int q = 0; q < G; q++) {
+            const int r = grp * G + q, tm = r / 4, i = r % 4;
+            const float m = big_m[q];
             float top = m;
             top = __builtin_fmaxf(top, dpp_move<0xB1>(top));
             top = __builtin_fmaxf(top, dpp_move<0x4E>(top));
             top = __builtin_fmaxf(top, dpp_move<0x141>(top));
             top = __builtin_fmaxf(top, dpp_move<0x140>(top));
             // a lane with no column block holds (-inf, 0) and adds 0 * 2^-inf = 0
-            float s = big_s[tm][i] * __builtin_amdgcn_exp2f(m - top);
+            float s = big_s[q] * __builtin_amdgcn_exp2f(m - top);
             s += dpp_move<0xB1>(s);
             s += dpp_move<0x4E>(s);
             s += dpp_move<0x141>(s);
             s += dpp_move<0x140>(s);
-            float f = __builtin_amdgcn_exp2f(in.shift[tm][i] - top) * (1.0f / s);
+            float f = __builtin_amdgcn_exp2f(out.shift[tm][i] - top) * (1.0f / s);
             f = failed ? __builtin_nanf("") : f;
-#pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                out.acc[tm][tn][i] = in.acc[tm][tn][i] * f;
-            }
+            detail::store_score_row(out.home, out.row0, out.col0, out, tm, i, f);
         }
     }
+    out.stored = true;
 }
 
 }  // namespace gernels
