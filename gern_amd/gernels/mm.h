@@ -164,9 +164,8 @@ __device__ __forceinline__ void write_acc(const MatrixF32 &m, int64_t x, int64_t
                     if (ADD) {
                         p[dr * ld] += t.acc[tm][tn][i];
                     } else {
-                        // written once, never re-read by this kernel: keep it out of L2
-                        // (neutral at 4096^3, 1-2 % at 8192^3 where C is 256 MB)
-                        __builtin_nontemporal_store(t.acc[tm][tn][i], p + dr * ld);
+                        // written once, never re-read by this kernel
+                        store_result4<kThroughStores>(m.data, (m.row - 1) * m.lda + m.col, (r0 + tm * 32 + dr) * m.lda + (c0 + tn * 32), t.acc[tm][tn][i]);
                     }
                 }
             }
@@ -703,7 +702,7 @@ __device__ __forceinline__ void write_acc_f32(const MatrixF32 &m, int64_t x, int
                     v = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
                     *reinterpret_cast<float4 *>(p) = v;
                 } else {
-                    store_streaming(p, v);
+                    store_result16<kThroughStores>(m.data, (m.row - 1) * m.lda + m.col, rr * m.lda + c0, v);
                 }
             } else {
                 const float e[4] = {v.x, v.y, v.z, v.w};

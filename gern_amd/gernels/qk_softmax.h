@@ -105,7 +105,7 @@ __device__ __forceinline__ void MatrixF32::store_row_block(int64_t x, int64_t y,
             const int64_t cc = c0 + 64 * g;
             const float4 val = make_float4(t.acc[g][0][i], t.acc[g][1][i], t.acc[g][2][i], t.acc[g][3][i]);
             if (vec_ok && cc + 3 < col) {
-                store_streaming(p + cc, val);
+                store_result16<kThroughStores>(data, (row - 1) * lda + col, rr * lda + cc, val);
             } else {
                 if (cc + 0 < col) p[cc + 0] = val.x;
                 if (cc + 1 < col) p[cc + 1] = val.y;

@@ -183,7 +183,7 @@ __device__ __forceinline__ void store_score_row(const MatrixF32 &m, int64_t x, i
         const float4 val = make_float4(t.acc[tm][4 * g + 0][i] * f, t.acc[tm][4 * g + 1][i] * f, t.acc[tm][4 * g + 2][i] * f,
                                        t.acc[tm][4 * g + 3][i] * f);
         if (cc + 3 < m.col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
-            store_streaming(p + cc, val);
+            store_result16<kThroughStores>(m.data, (m.row - 1) * m.lda + m.col, rr * m.lda + cc, val);
         } else {
             if (cc + 0 < m.col) p[cc + 0] = val.x;
             if (cc + 1 < m.col) p[cc + 1] = val.y;

@@ -47,6 +47,49 @@ __device__ __forceinline__ void store_streaming(float *p, const float4 &v) {
     __builtin_nontemporal_store(q, reinterpret_cast<f32x4_native *>(p));
 }
 
+// Stores of RESULTS, which the kernel does not read again: base[elem .. elem + 3]
+// (base[elem]) of a matrix that spans `span` elements from base.  They go out as
+// buffer stores that are written through to memory at once (agent scope): the
+// lines are then clean when the kernel ends, where ordinary and nontemporal
+// stores leave them for the write-back that closes every kernel.  POLICY is the
+// cache policy of the buffer instruction (1 = sc0, 2 = nt, 16 = sc1):
+//   kThroughStores           written through; for kernels that re-read nothing
+//                            from L2 (64 MiB of results, us per launch: write-only
+//                            kernel 11.1 -> 10.1, QK^T softmax tiles 22.4 -> 21.2,
+//                            row blocks 27.4 -> 24.6; the GEMMs: no difference)
+//   kThroughStreamingStores  written through and nontemporal; for kernels whose
+//                            inputs must stay in L2 for a neighbouring tile (blur
+//                            8192^2 over rotating buffers 91.2 -> 90.0 us, softmax
+//                            45.0 -> 44.5 us; written through only: 91.4 and 45.4,
+//                            and the blur on the same buffers 90 instead of 81 us)
+// Buffer addressing takes 32-bit byte offsets, so a matrix of 4 GiB or more
+// keeps nontemporal stores.
+constexpr int kThroughStores = 16;
+constexpr int kThroughStreamingStores = 18;
+
+template<int POLICY>
+__device__ __forceinline__ void store_result16(float *base, int64_t span, int64_t elem, const float4 &v) {
+    typedef unsigned int u32x4_native __attribute__((ext_vector_type(4)));
+    if ((uint64_t)span * 4u < 0xFFFFFFF0ull) {  // uniform
+        const __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(span * 4), 0x00020000);
+        const u32x4_native bits = {__builtin_bit_cast(unsigned int, v.x), __builtin_bit_cast(unsigned int, v.y),
+                                   __builtin_bit_cast(unsigned int, v.z), __builtin_bit_cast(unsigned int, v.w)};
+        __builtin_amdgcn_raw_buffer_store_b128(bits, desc, (int)(elem * 4), 0, POLICY);
+    } else {
+        store_streaming(base + elem, v);
+    }
+}
+
+template<int POLICY>
+__device__ __forceinline__ void store_result4(float *base, int64_t span, int64_t elem, float v) {
+    if ((uint64_t)span * 4u < 0xFFFFFFF0ull) {  // uniform
+        const __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(span * 4), 0x00020000);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), desc, (int)(elem * 4), 0, POLICY);
+    } else {
+        __builtin_nontemporal_store(v, base + elem);
+    }
+}
+
 template<int64_t R, int64_t C>
 __device__ __forceinline__ WaveTile<R, C> allocate_wave_tile() {
     return WaveTile<R, C>();
@@ -230,8 +273,8 @@ struct MatrixF32 {
                     // A result tile is written once and never read back by
                     // the kernel: a streaming (nontemporal) store keeps it
                     // from displacing the input rows that neighbouring tiles
-                    // are about to re-read from L2.
-                    store_streaming(p + lc, val);
+                    // are about to re-read from L2 (and it is written through).
+                    store_result16<kThroughStreamingStores>(data, (row - 1) * lda + col, rr * lda + y + lc, val);
                 } else {
                     if (lc + 0 < C && cc + 0 < col) p[lc + 0] = val.x;
                     if (lc + 1 < C && cc + 1 < col) p[lc + 1] = val.y;
@@ -278,7 +321,7 @@ struct MatrixF32 {
             hi = hi < col ? hi : col;
             const float4 val = t.v[r][0];
             if (vec_ok && cc >= lo && cc + 3 < hi) {
-                store_streaming(p + cc, val);
+                store_result16<kThroughStreamingStores>(data, (row - 1) * lda + col, rr * lda + cc, val);
             } else {
                 if (cc + 0 >= lo && cc + 0 < hi) p[cc + 0] = val.x;
                 if (cc + 1 >= lo && cc + 1 < hi) p[cc + 1] = val.y;
