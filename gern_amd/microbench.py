@@ -22,7 +22,8 @@ qk_phases         the same for the QK^T softmax tile kernel (gernels/qk_tiles.h)
 mfma_rate         a loop of nothing but v_mfma_f32_32x32x16_bf16 with changing
                   operands on every SIMD for about a millisecond: the sustained
                   matrix rate and clock of this GPU
-write_rate        a kernel that only writes 64 MiB (16-byte streaming stores):
+write_rate        a kernel that only writes 64 MiB (16-byte streaming stores, and
+                  16-byte stores written through to memory as the gernels use them):
                   the floor of any kernel that writes a 4096 x 4096 fp32 result
 
 Prints a table per probe on stdout.  These are measurements of the library's
@@ -144,6 +145,14 @@ extern "C" __global__ void __launch_bounds__(256) write_rate(f32x4_t *out, long 
     const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
     const f32x4_t v = {1.f, 2.f, 3.f, 4.f};
     if (i < n) __builtin_nontemporal_store(v, out + i);
+}
+// the same with stores that are written through to memory (the gernels' store_result16)
+extern "C" __global__ void __launch_bounds__(256) write_rate_through(float *out, long long n) {
+    typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const u32x4_t v = {0x3f800000u, 0x40000000u, 0x40400000u, 0x40800000u};
+    const __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc((void *)out, 0, (int)(n * 16), 0x00020000);
+    if (i < n) __builtin_amdgcn_raw_buffer_store_b128(v, desc, (int)(i * 16), 0, 16);
 }
 """
 
@@ -348,7 +357,7 @@ def qk_phases(gern_amd, torch):
 
 
 def mfma_rate(gern_amd, torch):
-    (k, _) = _compile(gern_amd, RATE_SRC, ["mfma_rate", "write_rate"])
+    (k, _, _) = _compile(gern_amd, RATE_SRC, ["mfma_rate", "write_rate", "write_rate_through"])
     sink = torch.zeros(16, device="cuda")
     stamps = torch.zeros((256, 4), dtype=torch.int64, device="cuda")
     iters = 6000  # x 8 MFMAs x 32 cycles x 2 wavefronts per SIMD: ~3.1 M cycles
@@ -368,14 +377,16 @@ def mfma_rate(gern_amd, torch):
 
 
 def write_rate(gern_amd, torch):
-    (_, k) = _compile(gern_amd, RATE_SRC, ["mfma_rate", "write_rate"])
+    (_, k, kt) = _compile(gern_amd, RATE_SRC, ["mfma_rate", "write_rate", "write_rate_through"])
     out = torch.zeros(16 * 1024 * 1024, device="cuda")  # 64 MiB
     n = C.c_longlong(out.numel() // 4)
     args = [C.c_void_p(out.data_ptr()), n]
     grid = ((out.numel() // 4 + 255) // 256, 1, 1)
-    us = _event_us(gern_amd, torch, lambda: _launch(gern_amd, k, grid, (256, 1, 1), args), 10, 100)
-    us = _event_us(gern_amd, torch, lambda: _launch(gern_amd, k, grid, (256, 1, 1), args), 10, 100)
-    print("write-only kernel, 64 MiB of 16-byte streaming stores: %.1f us per launch = %.0f GB/s" % (us, out.numel() * 4 / (us * 1e-6) / 1e9))
+    for name, kernel in (("16-byte streaming stores", k), ("16-byte stores written through to memory", kt)):
+        us = _event_us(gern_amd, torch, lambda: _launch(gern_amd, kernel, grid, (256, 1, 1), args), 10, 100)
+        us = _event_us(gern_amd, torch, lambda: _launch(gern_amd, kernel, grid, (256, 1, 1), args), 10, 100)
+        print("write-only kernel, 64 MiB of %s: %.1f us per launch = %.0f GB/s" % (name, us, out.numel() * 4 / (us * 1e-6) / 1e9))
+    assert float(out[1]) == 2.0 and float(out[-1]) == 4.0
 
 
 def main():
