@@ -229,6 +229,22 @@ def test_softmax_all_negative_rows_and_constant_rows(gpu, oracle):
     assert np.all(got[3] == np.float32(1.0 / 4096))
 
 
+# Results leave through buffer stores with 32-bit byte offsets; a matrix beyond 2 GiB has offsets with
+# the top bit set, one beyond 4 GiB takes the other store path.  Every element must be written either way.
+@pytest.mark.parametrize("rows", [150000, 270000])
+def test_softmax_results_beyond_2_and_4_gib(gpu, rows):
+    import torch
+    x = torch.randn((rows, 4096), device="cuda")
+    y = torch.full_like(x, float("nan"))
+    gpu.Softmax(4096)(x, y)
+    torch.cuda.synchronize()
+    assert int(torch.isnan(y).sum()) == 0
+    for lo in (0, rows // 2, rows - 64):
+        want = torch.softmax(x[lo:lo + 64].double(), dim=1)
+        assert float(((y[lo:lo + 64].double() - want).abs() / want).max()) < 1e-5, lo
+    assert float((y.sum(dim=1, dtype=torch.float64) - 1).abs().max()) < 1e-5
+
+
 @pytest.mark.parametrize("ncol", [1000, 4096])
 def test_softmax_rows_with_a_wide_range(gpu, oracle, ncol):
     # differences of more than 87 from the row maximum: exp leaves the range of
