@@ -60,6 +60,7 @@ def _load():
     pipes.gern_pipeline_kernel_name.restype = C.c_char_p
     pipes.gern_pipeline_kernel_name.argtypes = [vp]
     pipes.gern_pipeline_destroy.argtypes = [vp]
+    pipes.gern_pipeline_faults.argtypes = [vp, C.POINTER(i64)]
     pipes.gern_blur_chain_create.argtypes = [C.c_char_p, i64, i64, i64, C.c_int, C.c_int, C.POINTER(vp)]
     pipes.gern_blur_chain_run.argtypes = [vp, vp, i64, i64, i64, vp, i64, vp]
     pipes.gern_softmax_create.argtypes = [i64, i64, C.c_int, C.POINTER(vp)]
@@ -175,6 +176,13 @@ class _Pipeline:
     @property
     def kernel_name(self):
         return pipelines_lib().gern_pipeline_kernel_name(self.h).decode()
+
+    def faults(self):
+        """gern_pipeline_faults: waits for the device; what the kernels could only signal in their results
+        (QK tile kernel: wavefronts that gave up waiting, rows whose logits did not fit), read and cleared."""
+        n = C.c_int64(-1)
+        _check(pipelines_lib().gern_pipeline_faults(self.h, C.byref(n)))
+        return n.value
 
     def __del__(self):
         try:

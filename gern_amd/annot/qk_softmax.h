@@ -175,7 +175,7 @@ private:
 // (gernels::RowStatsExchange): device memory, all zeros before its first use.
 struct RowStatsExchangeLayout {
     void *entries;       // `capacity` entries of 8 bytes: rows (padded to the tile height) x pitch of them are used
-    void *state;         // two 32-bit words
+    void *state;         // four 32-bit words: launch number, workgroups done, wavefronts that gave up, rows that did not fit
     int32_t pitch;       // entries per row: at least the number of column blocks
     int32_t spin_limit;  // polls before a wavefront gives up
     int64_t capacity;

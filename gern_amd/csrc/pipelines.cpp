@@ -14,6 +14,7 @@
 
 #include <dlfcn.h>
 
+#include <cerrno>
 #include <cmath>
 #include <cstring>
 #include <algorithm>
@@ -51,6 +52,13 @@ std::string packageDir() {
     return ".";
 }
 
+// GERN_EXPERIMENTS=1 lets the environment change what the pipelines are built from (extra compiler
+// options, other band heights and wavefront counts): for measurements, never needed for results.
+bool experiments() {
+    const char *v = std::getenv("GERN_EXPERIMENTS");
+    return v != nullptr && std::string(v) == "1";
+}
+
 AbstractDataTypePtr f32(const std::string &name, annot::MatrixF32::Role role) {
     return AbstractDataTypePtr(new const annot::MatrixF32(name, role));
 }
@@ -76,6 +84,11 @@ struct gern_pipeline_s {
     // qk on 256 x 256 tiles: the memory through which the workgroups of a row block exchange row statistics
     bool qk_tiles = false;
     void *qk_scratch = nullptr;
+    // the exchange memory of the library (csrc/qk_no_alloc.hip) on this pipeline's GPU; null if it has none
+    void *qk_shared_scratch = nullptr;
+    bool qk_used_shared = false;      // a run went through qk_shared_scratch since the last gern_pipeline_faults
+    bool qk_default_period = true;    // built with the tag period every user of the shared memory agrees on
+    void *last_stream = nullptr;
     // parameter names
     std::vector<std::string> names;
 };
@@ -90,8 +103,9 @@ int64_t qkWaves(int64_t n) {
 // Generates (and, unless compile-only, loads) the program.
 int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_simd = 0, int xcd_band_rows = 0) {
     std::string include = "-I " + packageDir();
-    if (const char *extra = std::getenv("GERN_PIPELINE_EXTRA_OPTIONS")) {
-        include += std::string(" ") + extra;  // e.g. "-DNAME=value", for experiments
+    if (const char *extra = std::getenv("GERN_PIPELINE_EXTRA_OPTIONS"); extra != nullptr && experiments()) {
+        include += std::string(" ") + extra;  // e.g. "-DNAME=value"
+        p->qk_default_period = std::string(extra).find("GERN_QK_TAG_PERIOD") == std::string::npos;
     }
     try {
         if (flags & GERN_PIPELINE_COMPILE_ONLY) {
@@ -144,6 +158,10 @@ int finish(gern_pipeline_s *p, Composable program, int flags, int min_waves_per_
 }
 
 }  // namespace
+
+// csrc/qk_no_alloc.hip: the address of the library's exchange memory on the current GPU (looked up, once per
+// GPU, on the first call).  Weak: a build of this file without that object has no such memory.
+extern "C" __attribute__((weak, visibility("hidden"))) int gern_detail_qk_shared_scratch(void **out);
 
 extern "C" {
 
@@ -216,10 +234,10 @@ int gern_blur_chain_create(const char *pattern, int64_t stride, int64_t tile_row
         // another XCD), and the eight XCDs stream through one 16 MiB window of an 8192-wide image together
         // instead of through eight places 32 MiB apart: 8192^2 x,y,x over rotating buffers 92.6 -> 90.3 us,
         // same buffers 86 -> 78-86 us (measured in one process; bands of 8 rows of tiles 89.8 us, of 32 and
-        // more 94-105 us, one tile row per band 108 us).  GERN_BLUR_BAND_ROWS overrides it for experiments
-        // (0 = one contiguous run of tiles per XCD).
+        // more 94-105 us, one tile row per band 108 us).  With GERN_EXPERIMENTS=1, GERN_BLUR_BAND_ROWS
+        // overrides it (0 = one contiguous run of tiles per XCD).
         int band_rows = (int)std::max<int64_t>(1, 64 / tile_rows);
-        if (const char *v = std::getenv("GERN_BLUR_BAND_ROWS")) {
+        if (const char *v = std::getenv("GERN_BLUR_BAND_ROWS"); v != nullptr && experiments()) {
             band_rows = std::max(0, std::atoi(v));
         }
         int rc = finish(p.get(), program, flags, 0, band_rows);
@@ -278,7 +296,7 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
             break;
         }
     }
-    if (const char *forced = std::getenv("GERN_SOFTMAX_WAVES")) {
+    if (const char *forced = std::getenv("GERN_SOFTMAX_WAVES"); forced != nullptr && experiments()) {
         waves = std::atoll(forced);
         if ((waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) || ncol % (4 * waves) != 0) {
             return fail("GERN_SOFTMAX_WAVES must be 1, 2, 4, 8 or 16 and divide the row into 16-byte pieces");
@@ -584,6 +602,11 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
                 gern_hip_last_error(msg.data(), msg.size());
                 return fail("gern_qk_softmax_create: " + msg);
             }
+            // Look the library's own exchange memory up now (the runtime loads the library's code object at
+            // the first lookup on a GPU), so that gern_qk_softmax_run_no_alloc never does.
+            if (gern_detail_qk_shared_scratch != nullptr && gern_detail_qk_shared_scratch(&p->qk_shared_scratch) != 0) {
+                return 1;  // message set
+            }
         }
     } catch (const std::exception &e) {
         return fail(e.what());
@@ -595,12 +618,22 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
 namespace {
 
 // Polls before a wavefront of the tile kernel gives up on the other tiles of its
-// row block (a poll takes a microsecond or two); GERN_QK_SPIN_LIMIT overrides it.
-int32_t qkSpinLimit() {
-    if (const char *forced = std::getenv("GERN_QK_SPIN_LIMIT")) {
-        return (int32_t)std::atol(forced);
+// row block (a poll takes a microsecond or two); GERN_QK_SPIN_LIMIT, a whole
+// number from 0 to 2^31 - 1, overrides it.  False: the variable holds something else.
+bool qkSpinLimit(int32_t *limit) {
+    *limit = 1 << 18;
+    const char *forced = std::getenv("GERN_QK_SPIN_LIMIT");
+    if (forced == nullptr) {
+        return true;
     }
-    return 1 << 18;
+    char *end = nullptr;
+    errno = 0;
+    const long long v = std::strtoll(forced, &end, 10);
+    if (end == forced || *end != '\0' || errno != 0 || v < 0 || v > 0x7FFFFFFFll) {
+        return false;
+    }
+    *limit = (int32_t)v;
+    return true;
 }
 
 }  // namespace
@@ -633,6 +666,7 @@ __attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeli
     hip::MatrixF32 s{S, M, N, N};
     try {
         p->runner->setStream(stream);
+        p->last_stream = stream;
         if (!p->qk_tiles) {
             p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"scale", &scale}});
             return 0;
@@ -644,7 +678,12 @@ __attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeli
         if (scratch == nullptr || padded_rows * pitch > capacity) {
             return fail(name + ": M x N needs more than GERN_QK_SCRATCH_BYTES of exchange memory (M up to 16384 at 4096 keys)");
         }
-        annot::RowStatsExchangeLayout exchange{static_cast<char *>(scratch) + 256, scratch, (int32_t)pitch, qkSpinLimit(), capacity};
+        int32_t spin_limit = 0;
+        if (!qkSpinLimit(&spin_limit)) {
+            return fail(name + ": GERN_QK_SPIN_LIMIT must be a whole number from 0 to 2147483647");
+        }
+        p->qk_used_shared = p->qk_used_shared || scratch != p->qk_scratch;
+        annot::RowStatsExchangeLayout exchange{static_cast<char *>(scratch) + 256, scratch, (int32_t)pitch, spin_limit, capacity};
         p->runner->evaluate({{"Q", &q}, {"K", &k}, {"S", &s}, {"exchange", &exchange}, {"scale", &scale}});
     } catch (const std::exception &e) {
         return fail(e.what());
@@ -656,6 +695,65 @@ int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, f
                         float scale, void *stream) {
     return gern_detail_qk_softmax_run(p, Q, K, S, M, N, scale, p != nullptr ? p->qk_scratch : nullptr, stream,
                                       "gern_qk_softmax_run");
+}
+
+// The library's exchange memory as gern_qk_softmax_create found it for this pipeline (csrc/qk_no_alloc.hip
+// calls this; it never looks anything up in a run).  Null with a message when the pipeline may not use it.
+__attribute__((visibility("hidden"))) void *gern_detail_qk_shared_of(gern_pipeline p) {
+    if (p == nullptr || p->kind != gern_pipeline_s::QK_SOFTMAX) {
+        fail("gern_qk_softmax_run_no_alloc: bad pipeline");
+        return nullptr;
+    }
+    if (p->qk_tiles && !p->qk_default_period) {
+        // every user of the shared memory must agree on when the launch number wraps around
+        fail("gern_qk_softmax_run_no_alloc: the pipeline was built with another GERN_QK_TAG_PERIOD than the library's exchange memory is used with");
+        return nullptr;
+    }
+    if (p->qk_tiles && p->qk_shared_scratch == nullptr) {
+        fail("gern_qk_softmax_run_no_alloc: the pipeline has no access to the library's exchange memory (created compile-only?)");
+        return nullptr;
+    }
+    return p->qk_tiles ? p->qk_shared_scratch : static_cast<void *>(p);  // the other kernel needs none: any non-null value
+}
+
+int gern_pipeline_faults(gern_pipeline p, int64_t *count) {
+    if (p == nullptr || count == nullptr) {
+        return fail("gern_pipeline_faults: null argument");
+    }
+    *count = 0;
+    try {
+        for (Runner *r : {p->runner.get(), p->exact.get(), p->tail.get()}) {
+            if (r != nullptr) {
+                *count += r->ldsOverflows();  // waits for the device; zero for kernels without the LDS allocator
+            }
+        }
+    } catch (const std::exception &e) {
+        return fail(e.what());
+    }
+    if (!p->qk_tiles || !p->runner) {
+        return 0;
+    }
+    if (gern_hip_sync() != 0) {
+        std::string msg(gern_hip_last_error(nullptr, 0) + 1, '\0');
+        gern_hip_last_error(msg.data(), msg.size());
+        return fail("gern_pipeline_faults: " + msg);
+    }
+    // words 2 and 3 of the exchange's state: wavefronts that gave up, (row, column block) pairs that did not fit
+    for (void *scratch : {p->qk_scratch, p->qk_used_shared ? p->qk_shared_scratch : nullptr}) {
+        if (scratch == nullptr) {
+            continue;
+        }
+        uint32_t words[2] = {0, 0};
+        char *at = static_cast<char *>(scratch) + 8;
+        if (gern_hip_memcpy_d2h(words, at, sizeof(words)) != 0 || ((words[0] | words[1]) != 0 && gern_hip_memset(at, 0, sizeof(words)) != 0)) {
+            std::string msg(gern_hip_last_error(nullptr, 0) + 1, '\0');
+            gern_hip_last_error(msg.data(), msg.size());
+            return fail("gern_pipeline_faults: " + msg);
+        }
+        *count += (int64_t)words[0] + (int64_t)words[1];
+    }
+    p->qk_used_shared = false;
+    return 0;
 }
 
 // User-level GEMM schedules over the LDS-staged matrices (annot/lds_matrix.h), as the reference's

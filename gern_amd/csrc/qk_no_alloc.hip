@@ -3,7 +3,8 @@
 // the workgroups of the tile kernel exchange row statistics (gernels/qk_tiles.h)
 // comes from a device array of this library instead of the pipeline's own
 // allocation.  Every GPU holds its own copy of the array, at its own address,
-// from the moment the array is first looked up until the process ends.
+// from the moment the array is first looked up (when the first tile-kernel
+// pipeline is created on that GPU) until the process ends.
 #include "gern_pipelines.h"
 
 #include <hip/hip_runtime.h>
@@ -17,6 +18,7 @@ __attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeli
                                                                      int64_t M, int64_t N, float scale, void *scratch, void *stream,
                                                                      const char *who);
 __attribute__((visibility("hidden"))) int gern_detail_fail(const char *message);
+__attribute__((visibility("hidden"))) void *gern_detail_qk_shared_of(gern_pipeline p);
 }
 
 namespace {
@@ -58,10 +60,16 @@ int scratchOfCurrentDevice(void **out) {
 
 }  // namespace
 
+// For gern_qk_softmax_create (csrc/pipelines.cpp): set-up, once per GPU, with that GPU current.
+extern "C" __attribute__((visibility("hidden"))) int gern_detail_qk_shared_scratch(void **out) {
+    return scratchOfCurrentDevice(out);
+}
+
+// The run itself looks nothing up: the address was found when the pipeline was created.
 extern "C" int gern_qk_softmax_run_no_alloc(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M, int64_t N,
                                             float scale, void *stream) {
-    void *ptr = nullptr;
-    if (scratchOfCurrentDevice(&ptr) != 0) {
+    void *ptr = gern_detail_qk_shared_of(p);
+    if (ptr == nullptr) {
         return 1;
     }
     return gern_detail_qk_softmax_run(p, Q, K, S, M, N, scale, ptr, stream, "gern_qk_softmax_run_no_alloc");

@@ -412,29 +412,19 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         __builtin_amdgcn_s_barrier();
     };
 
-    // Diagnostic builds only (gern_amd.microbench, results are wrong): -DGERN_MM_ONLY=1 moves the
-    // data and computes nothing, -DGERN_MM_ONLY=2 computes every stage on what the first two loaded.
-#ifndef GERN_MM_ONLY
-#define GERN_MM_ONLY 0
-#endif
-    constexpr bool kCompute = GERN_MM_ONLY != 1, kReload = GERN_MM_ONLY != 2;
     issue(0, stage_even);
     arrive();
     for (int kt = 0; kt < nk; kt += 2) {
-        if (kt + 1 < nk && (kReload || kt == 0)) {
+        if (kt + 1 < nk) {
             issue(kt + 1, stage_odd);
         }
-        if (kCompute) {
-            compute(stage_even);
-        }
+        compute(stage_even);
         arrive();
         if (kt + 1 < nk) {
-            if (kt + 2 < nk && kReload) {
+            if (kt + 2 < nk) {
                 issue(kt + 2, stage_even);
             }
-            if (kCompute) {
-                compute(stage_odd);
-            }
+            compute(stage_odd);
             arrive();
         }
     }
@@ -1058,10 +1048,7 @@ __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, float, 
         // LDS reads of the next step.  Unrolling all sixteen makes the compiler
         // hoist every read and spread over 384 registers (measured: 40 instead
         // of 72 TFLOP/s).
-#ifndef GERN_FMA_UNROLL
-#define GERN_FMA_UNROLL 4
-#endif
-#pragma unroll GERN_FMA_UNROLL
+#pragma unroll 4
         for (int k = 0; k < kFmaBK; k++) {
             const float4 a0 = *reinterpret_cast<const float4 *>(a_lds + k * kFmaLd + ty * 4);
             const float4 a1 = *reinterpret_cast<const float4 *>(a_lds + k * kFmaLd + 64 + ty * 4);

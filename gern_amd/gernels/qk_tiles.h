@@ -56,17 +56,18 @@
 // of its own row block, and those never wait for a later one.  The wait is
 // bounded all the same: after spin_limit polls a wavefront gives up and stores
 // NaN in its rows.  Logits beyond +-32767 in log2 units (22 000 in natural
-// units) do not fit an entry; their rows come out as NaN.
+// units) do not fit an entry; their rows come out as NaN.  Neither goes
+// unnoticed by the host: state[2] counts the wavefronts that gave up and
+// state[3] the (row, column block) pairs whose shift did not fit or whose
+// logits were not all numbers, for the host to read and clear after the launch (the reference
+// checks for an error after every launch,
+// include/gern/codegen/helpers/check_last_error.h:7-18).
 //
 // Two launches that use the same exchange must not overlap in time.
 #pragma once
 
 #include "gernels/mm.h"
 #include "gernels/softmax.h"
-
-#ifndef GERN_QK_SLEEP
-#define GERN_QK_SLEEP 2
-#endif
 
 namespace gernels {
 
@@ -83,7 +84,9 @@ constexpr unsigned int kRowStatsTagPeriod = GERN_QK_TAG_PERIOD;
 // layout): `entries` holds `capacity` entries of 8 bytes, at least rows x
 // pitch for the padded row count of the launch, pitch >= the number of column
 // blocks; state[0] is the launch number, state[1] counts the workgroups that
-// are done.  All of it starts as zeros.
+// are done, state[2] the wavefronts that gave up waiting and state[3] the
+// (row, column block) pairs whose logits did not fit an entry (the host reads
+// and clears these two).  All of it starts as zeros.
 struct RowStatsSession {
     unsigned long long *entries;
     unsigned int *state;
@@ -387,10 +390,7 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
     // Rows per lane and pipeline step (slot r = 4 tm + i is row 16 tm + i of the lane's eight rows).  Measured
     // at 4096 x 4096 x 128 in one process: 8 (one exchange for all rows) 24.3 us, 4 (the two halves) 21.7 us,
     // 1 (row by row) 23.6 us.
-#ifndef GERN_QK_GROUP
-#define GERN_QK_GROUP 4
-#endif
-    constexpr int G = GERN_QK_GROUP;
+    constexpr int G = 4;
     static_assert(G == 1 || G == 2 || G == 4 || G == 8, "group size");
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
@@ -403,6 +403,7 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
     const u64 tag = ex.tag;
     out.unit = 1.0f;
     out.valid_cols = in.valid_cols;
+    unsigned int unfit = 0;  // rows of this lane whose shift does not fit an entry (the same in all sixteen lanes of a row)
 #pragma unroll
     for (int grp = 0; grp < 8 / G; grp++) {
 #pragma unroll
@@ -438,7 +439,8 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
             const float a = flip ? -unit : unit;
             // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
             // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
-            const float shift = __builtin_fminf(__builtin_fmaxf(__builtin_floorf(m * a), -32768.0f), 32767.0f);
+            const float whole = __builtin_floorf(m * a);
+            const float shift = __builtin_fminf(__builtin_fmaxf(whole, -32768.0f), 32767.0f);
             float s = 0.f;
 #pragma unroll
             for (int tn = 0; tn < 16; tn++) {
@@ -457,6 +459,8 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
             s += dpp_move<0x140>(s);
             out.shift[tm][i] = shift;
             out.sum[tm][i] = s;
+            // the largest logit beyond an entry's range or not a number, or a logit that is not a number
+            unfit += (whole != shift || s != s) ? 1u : 0u;
         }
         {
             // lane j < G of each 16-lane row publishes slot grp * G + j
@@ -474,6 +478,10 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
             }
         }
     }
+    if (unfit != 0u && jl == 0) {  // never, for logits that fit: one lane per 16-lane row reports its rows
+        __hip_atomic_fetch_add(ex.state + 3, unfit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    bool gave_up = false;
 #pragma unroll
     for (int grp = 0; grp < 8 / G; grp++) {
         // Lane j collects column block j (j + 16, ...) for the G rows it holds of this group.
@@ -509,7 +517,7 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
                     failed = true;
                     break;
                 }
-                __builtin_amdgcn_s_sleep(GERN_QK_SLEEP);
+                __builtin_amdgcn_s_sleep(2);  // 0 to 32 measure the same
             }
             if (b < nbj) {
 #pragma unroll
@@ -521,7 +529,11 @@ __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> 
                 }
             }
         }
+        gave_up = gave_up || failed;
         if (grp == 8 / G - 1) {
+            if (gave_up && lane == 0) {  // wave-uniform condition
+                __hip_atomic_fetch_add(ex.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
         }
 #pragma unroll

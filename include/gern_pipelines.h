@@ -124,7 +124,11 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
  * (launch them on one stream, or order the streams).  A wavefront that waits
  * in vain for the rest of its row block (after a second or so: the launch
  * shares the GPU with something that keeps its partners from starting) stores
- * NaN in its rows, and so does a row whose logits exceed 22 000 in magnitude.
+ * NaN in its rows, and so does a row whose logits exceed 22 000 in magnitude;
+ * the run still returns 0 (it is asynchronous), and gern_pipeline_faults
+ * reports both afterwards.  The environment variable GERN_QK_SPIN_LIMIT (a
+ * whole number from 0 to 2^31 - 1; anything else makes the run fail) sets the
+ * number of polls before a wavefront gives up.
  * Other D (or GERN_PIPELINE_QK_ROW_BLOCKS): sixteen whole rows of S per
  * workgroup, logits in accumulators, no device memory besides Q, K and S.
  * No counterpart in the reference (it has no bf16 and no matrix-core path);
@@ -149,16 +153,38 @@ int gern_gemm_schedule_run(gern_pipeline p, const float *A, const float *B, floa
 
 /* gern_qk_softmax_run with the exchange memory taken from a device array of
  * this library (GERN_QK_SCRATCH_BYTES, one copy per GPU, held from the first
- * call on that GPU until the process ends) instead of the pipeline's own
- * allocation: the call allocates nothing on the device, for callers that must
- * not (a stream under HIP graph capture, a serving loop that forbids it).
+ * gern_qk_softmax_create of a tile-kernel pipeline on that GPU until the
+ * process ends) instead of the pipeline's own allocation: the call allocates
+ * nothing on the device and looks nothing up (gern_qk_softmax_create found the
+ * array, which is when the runtime loads this library's device code), for
+ * callers that must not allocate (a stream under HIP graph capture, a serving
+ * loop that forbids it).
  * Same arguments, same limits (M x N must fit GERN_QK_SCRATCH_BYTES), same
  * results.  All pipelines of a process share the array of a GPU: calls of this
  * function that overlap in time on one GPU race (launch them on one stream,
- * or order the streams); calls of gern_qk_softmax_run do not touch it.
+ * or order the streams); calls of gern_qk_softmax_run do not touch it.  A
+ * pipeline built with another launch-tag period than the library's default
+ * (an experiment option) is refused: all users of the array must agree on it.
  * No counterpart in the reference. */
 int gern_qk_softmax_run_no_alloc(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S,
                                  int64_t M, int64_t N, float scale, void *stream);
+
+/* What the kernels of the pipeline could not do and could only signal in
+ * their results, since a run returns before they execute.  Waits for the
+ * device, then stores in *count, and clears, the sum of
+ *   - wavefronts of the QK^T softmax tile kernel that gave up waiting for
+ *     the rest of their row block (their rows of S hold NaN),
+ *   - (row, block of 256 keys) pairs of that kernel whose largest logit is
+ *     beyond +-22 000 or not a number (those rows of S hold NaN),
+ *     both over all runs of this pipeline since the last call (runs through
+ *     gern_qk_softmax_run_no_alloc count in one place per GPU, shared with
+ *     the other pipelines that use it),
+ *   - requests that the LDS allocator of a gern_gemm_schedule pipeline could
+ *     not meet (not cleared: a count over the life of the pipeline).
+ * 0 means every result is what the pipeline computes.  Takes the place of the
+ * reference's check after each launch,
+ * include/gern/codegen/helpers/check_last_error.h:7-18. */
+int gern_pipeline_faults(gern_pipeline p, int64_t *count);
 
 /* The generated device source (owned by the pipeline, valid until destroy).
  * A pipeline that holds more than one kernel (the GEMMs) reports the one its

@@ -274,10 +274,26 @@ def _run_gemm(gpu, variant, A, B, C0=None, general_only=False):
     return dC.cpu().numpy()
 
 
+def _assert_gemm_close(got, want, A, B, tol, rows=None, c0=None, what=None):
+    """Two bounds on got - want (got, want: the rows `rows` of the product of the VALUES A and B):
+    norm-wise, max |got - want| <= tol * max |want|, and element by element,
+    |got - want|_ij <= tol * (|A| |B| (+ |C0|))_ij in fp64 -- the scale of the rounding errors of THAT
+    dot product, so an element near zero may not be wrong by more than its own terms allow."""
+    lo, hi = (0, A.shape[0]) if rows is None else rows
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape == (hi - lo, B.shape[1]), (got.shape, want.shape, what)
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < tol, what
+    scale = np.abs(A[lo:hi].astype(np.float64)) @ np.abs(B.astype(np.float64))
+    if c0 is not None:
+        scale = scale + np.abs(c0[lo:hi].astype(np.float64))
+    excess = np.abs(got - want) - tol * scale
+    assert np.all(excess <= 0), (what, float(excess.max()), np.unravel_index(int(excess.argmax()), excess.shape))
+
+
 def test_gemm_f32_golden_and_known_answers(gpu, oracle, golden):
     got = _run_gemm(gpu, "f32", golden["gemm_A"], golden["gemm_B"])
     want = golden["gemm_C"]
-    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(24)
+    _assert_gemm_close(got, want, golden["gemm_A"], golden["gemm_B"], 1e-4 * np.sqrt(golden["gemm_A"].shape[1]))
     # test/test-cpu-mm.cpp: ascending 10x10, exact small integers
     a = golden["gemm_asc_A"]
     assert np.array_equal(_run_gemm(gpu, "f32", a, a), golden["gemm_asc_C"])
@@ -292,17 +308,17 @@ def test_gemm_f32_matches_oracle(gpu, oracle, M, N, K, general_only):
     B = oracle.uniform((K, N), 2, -1.0, 1.0)
     got = _run_gemm(gpu, "f32", A, B, general_only=general_only)
     want = oracle.gemm_f32(A, B)
-    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(K)
+    _assert_gemm_close(got, want, A, B, 1e-4 * np.sqrt(K))
 
 
 @pytest.mark.parametrize("general_only", [False, True])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (200, 136, 72), (512, 384, 256), (3, 2, 8), (130, 260, 1032)])
 def test_gemm_bf16_matches_oracle(gpu, oracle, M, N, K, general_only):
-    ab, _ = oracle.to_bf16(oracle.uniform((M, K), 1, -1.0, 1.0))
-    bb, _ = oracle.to_bf16(oracle.uniform((K, N), 2, -1.0, 1.0))
+    ab, av = oracle.to_bf16(oracle.uniform((M, K), 1, -1.0, 1.0))
+    bb, bv = oracle.to_bf16(oracle.uniform((K, N), 2, -1.0, 1.0))
     got = _run_gemm(gpu, "bf16", ab, bb, general_only=general_only)
     want = oracle.gemm_bf16(ab, bb)
-    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
+    _assert_gemm_close(got, want, av, bv, 1e-2)
     # exact small integers: products and sums are exact in fp32 in any order
     ai = np.random.RandomState(1).randint(-4, 5, size=(M, K)).astype(np.float32)
     bi = np.random.RandomState(2).randint(-4, 5, size=(K, N)).astype(np.float32)
@@ -339,15 +355,17 @@ def test_gemm_bf16_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     want = ai.astype(np.float64) @ bi.astype(np.float64) + (0 if overwrite else c0)
     assert np.array_equal(dC.cpu().numpy().astype(np.float64), want)
     # and ordinary values against the oracle
-    ab, _ = oracle.to_bf16(oracle.uniform((M, K), 21, -1.0, 1.0))
-    bb, _ = oracle.to_bf16(oracle.uniform((K, N), 22, -1.0, 1.0))
+    ab, av = oracle.to_bf16(oracle.uniform((M, K), 21, -1.0, 1.0))
+    bb, bv = oracle.to_bf16(oracle.uniform((K, N), 22, -1.0, 1.0))
     dC = torch.zeros((M, N), dtype=torch.float32, device="cuda")
     g(_dev(ab.view(np.int16)), _dev(bb.view(np.int16)), dC)
     torch.cuda.synchronize()
     rows = (max(M - 2, 0), M)
     want = oracle.gemm_bf16(ab, bb, rows=rows)[rows[0]:rows[1]]
-    got = dC.cpu().numpy()[rows[0]:rows[1]]
-    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-2
+    got = dC.cpu().numpy()
+    _assert_gemm_close(got[rows[0]:rows[1]], want, av, bv, 1e-2, rows=rows)
+    # every element against fp64 of the same bf16 values
+    _assert_gemm_close(got, av.astype(np.float64) @ bv.astype(np.float64), av, bv, 1e-2)
 
 
 # fp32 shapes with K >= 4 take the eight-wavefront kernel on the fp32
@@ -386,9 +404,8 @@ def test_gemm_f32_whole_tile_kernel(gpu, oracle, M, N, K, overwrite):
     got = dC.cpu().numpy()
     rows = (max(M - 2, 0), M)
     want = oracle.gemm_f32(A, B, rows=rows)[rows[0]:rows[1]]
-    assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(K)
-    want64 = A.astype(np.float64) @ B.astype(np.float64)
-    assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(K)
+    _assert_gemm_close(got[rows[0]:rows[1]], want, A, B, 1e-4 * np.sqrt(K), rows=rows)
+    _assert_gemm_close(got, A.astype(np.float64) @ B.astype(np.float64), A, B, 1e-4 * np.sqrt(K))
 
 
 # The matrix-core fp32 kernel reads rows of A in whole 16-byte pieces; a K
@@ -429,9 +446,8 @@ def test_gemm_user_schedules_match_oracle(gpu, oracle, schedule):
     got = dC.cpu().numpy()
     for rows in ((0, 8), (60, 68), (n - 4, n)):
         want = oracle.gemm_f32(A, B, rows=rows)[rows[0]:rows[1]]
-        assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < 1e-4 * np.sqrt(n)
-    want64 = A.astype(np.float64) @ B.astype(np.float64)
-    assert np.max(np.abs(got - want64)) / np.max(np.abs(want64)) < 1e-4 * np.sqrt(n)
+        _assert_gemm_close(got[rows[0]:rows[1]], want, A, B, 1e-4 * np.sqrt(n), rows=rows)
+    _assert_gemm_close(got, A.astype(np.float64) @ B.astype(np.float64), A, B, 1e-4 * np.sqrt(n))
 
 
 @pytest.mark.parametrize("variant", ["f32", "bf16"])
@@ -444,21 +460,26 @@ def test_gemm_accumulates_into_c(gpu, oracle, variant):
         bb, bv = oracle.to_bf16(B)
         got = _run_gemm(gpu, variant, ab, bb, C0)
         want = C0 + oracle.gemm_f32(av, bv)
+        A, B = av, bv
     else:
         got = _run_gemm(gpu, variant, A, B, C0)
         want = oracle.gemm_f32(A, B, C_in=C0)
-    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 1e-4
+    _assert_gemm_close(got, want, A, B, 1e-4, c0=C0)
 
 
-@pytest.mark.parametrize("variant,tol", [("f32", 1e-4 * 64), ("bf16", 1e-2)])
-def test_gemm_full_size(gpu, oracle, variant, tol):
+# general_only: the kernels that take every shape (fp32: vector-ALU FMAs, the kernel BASELINE's config 4a
+# names; bf16: the four-wavefront kernel that stages through registers) on the full-size product too.
+@pytest.mark.parametrize("variant,tol,general_only", [("f32", 1e-4 * 64, False), ("f32", 1e-4 * 64, True),
+                                                      ("bf16", 1e-2, False), ("bf16", 1e-2, True)])
+def test_gemm_full_size(gpu, oracle, variant, tol, general_only):
     M = N = K = 4096
     A = oracle.uniform((M, K), 4, -1.0, 1.0)
     B = oracle.uniform((K, N), 5, -1.0, 1.0)
+    av, bv = A, B
     if variant == "bf16":
         A, av = oracle.to_bf16(A)
         B, bv = oracle.to_bf16(B)
-    got = _run_gemm(gpu, variant, A, B)
+    got = _run_gemm(gpu, variant, A, B, general_only=general_only)
     # 64 whole rows against the oracle (every column, the last ones included):
     # the first and last rows of the first and last 256-row tiles, both sides of
     # two tile seams, of a wavefront seam and of an MFMA-tile seam inside a tile
@@ -466,11 +487,10 @@ def test_gemm_full_size(gpu, oracle, variant, tol):
     assert sum(b - a for a, b in bands) == 64
     for rows in bands:
         want = (oracle.gemm_bf16(A, B, rows=rows) if variant == "bf16" else oracle.gemm_f32(A, B, rows=rows))[rows[0]:rows[1]]
-        assert np.max(np.abs(got[rows[0]:rows[1]] - want)) / np.max(np.abs(want)) < tol, rows
+        _assert_gemm_close(got[rows[0]:rows[1]], want, av, bv, tol, rows=rows, what=rows)
     # Freivalds-style check of the whole product: C r == A (B r) in fp64
     r = np.random.RandomState(9).randint(0, 2, size=(N,)).astype(np.float64)
-    a64 = av.astype(np.float64) if variant == "bf16" else A.astype(np.float64)
-    b64 = bv.astype(np.float64) if variant == "bf16" else B.astype(np.float64)
+    a64, b64 = av.astype(np.float64), bv.astype(np.float64)
     lhs = got.astype(np.float64) @ r
     rhs = a64 @ (b64 @ r)
     assert np.max(np.abs(lhs - rhs)) / np.max(np.abs(rhs)) < 1e-4
@@ -512,12 +532,15 @@ def test_gemm_rejects_unsupported_bf16_shapes(gpu):
 
 
 # ------------------------------------------------------- QK^T -> softmax ----
-def _run_qk(gpu, qb, kb, scale, max_keys, flags=0):
+def _run_qk(gpu, qb, kb, scale, max_keys, flags=0, faults=0):
+    """One run on a fresh pipeline; the pipeline must report `faults` afterwards (None: not looked at)."""
     import torch
     p = gpu.QKSoftmax(qb.shape[1], max_keys, flags=flags)
     S = torch.full((qb.shape[0], kb.shape[0]), float("nan"), dtype=torch.float32, device="cuda")
     p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, scale)
     torch.cuda.synchronize()
+    if faults is not None:
+        assert p.faults() == faults
     return S.cpu().numpy()
 
 
@@ -566,18 +589,45 @@ def test_qk_softmax_tile_kernel_over_changing_shapes_and_scales(gpu, oracle):
         want = oracle.qk_softmax(qb, kb, np.float32(scale))
         assert np.max(np.abs(got - want) / want) < 1e-2, (M, N, scale)
         assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5), (M, N, scale)
+    assert p.faults() == 0
+
+
+# More workgroups than the GPU holds at once: 512 and 1024 tiles of 256 x 256 on 256 compute units, one
+# workgroup each.  The workgroups of a row block wait for one another, so this only works if a row block's
+# workgroups are dispatched together and ahead of the next row block's; nobody may give up waiting.
+@pytest.mark.parametrize("M", [8192, 16384])
+def test_qk_softmax_tile_kernel_with_more_workgroups_than_compute_units(gpu, oracle, M):
+    import torch
+    N, D = 4096, 128
+    qb, _ = oracle.to_bf16(oracle.normal((M, D), 81))
+    kb, _ = oracle.to_bf16(oracle.normal((N, D), 82))
+    scale = np.float32(1.0 / np.sqrt(D))
+    p = gpu.QKSoftmax(D, N)
+    assert "view_score_tile" in p.source
+    S = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, scale)
+    torch.cuda.synchronize()
+    assert p.faults() == 0
+    assert int(torch.isnan(S).sum()) == 0
+    assert float((S.sum(dim=1, dtype=torch.float64) - 1).abs().max()) < 1e-5
+    for r0 in (0, M // 2 + 250, M - 16):  # first, last, and across a seam of row blocks in the second half of the launch
+        got = S[r0:r0 + 16].cpu().numpy()
+        want = oracle.qk_softmax(qb, kb, scale, rows=(r0, r0 + 16))[r0:r0 + 16]
+        assert np.max(np.abs(got - want) / want) < 1e-2, r0
 
 
 def test_qk_softmax_tile_kernel_launch_number_wraps_around(gpu, oracle, monkeypatch):
     # A tag is the launch number; when the number wraps around, the last
     # workgroup of that launch clears every entry, so the entries that a tall
     # launch left behind one period ago are not taken for those of the current
-    # one.  The period is 2^32 - 1 launches; this pipeline is built with 1000.
+    # one.  The period is 65535 launches; this pipeline is built with 1000.
     import torch
     D = 64
+    monkeypatch.setenv("GERN_EXPERIMENTS", "1")
     monkeypatch.setenv("GERN_PIPELINE_EXTRA_OPTIONS", "-DGERN_QK_TAG_PERIOD=1000u")
     p = gpu.QKSoftmax(D, 512)
     monkeypatch.delenv("GERN_PIPELINE_EXTRA_OPTIONS")
+    monkeypatch.delenv("GERN_EXPERIMENTS")
     big = (oracle.to_bf16(oracle.normal((600, D), 71))[0], oracle.to_bf16(oracle.normal((512, D), 72))[0])
     small = (oracle.to_bf16(oracle.normal((8, D), 73))[0], oracle.to_bf16(oracle.normal((256, D), 74))[0])
     scale = np.float32(0.125)
@@ -596,6 +646,11 @@ def test_qk_softmax_tile_kernel_launch_number_wraps_around(gpu, oracle, monkeypa
     assert np.max(np.abs(run(*small, 1000) - want_small) / want_small) < 1e-2  # past the wrap: launch number 3 again
     for times in (1, 1, 1, 995, 3):                                            # launch numbers 3, 4, 5, ..., across the next wrap
         assert np.max(np.abs(run(*big, times) - want_big) / want_big) < 1e-2
+    assert p.faults() == 0
+    # the library's own exchange memory is shared by pipelines that all wrap at the default period: this one may not use it
+    S = torch.zeros((8, 256), dtype=torch.float32, device="cuda")
+    with pytest.raises(gpu.GernError, match="GERN_QK_TAG_PERIOD"):
+        p(_dev(small[0].view(np.int16)), _dev(small[1].view(np.int16)), S, scale, no_alloc=True)
 
 
 def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, monkeypatch):
@@ -620,11 +675,53 @@ def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, mo
     assert np.all(np.abs(got[~bad] - want[~bad]) / want[~bad] < 1e-2)
     # NaNs come as whole 256-column pieces of rows (one wavefront's rows of one tile)
     assert np.array_equal(bad, np.repeat(bad[:, ::256], 256, axis=1))
+    # the host learns of it without scanning S: one count per wavefront that gave up (32 rows x 256 columns
+    # each), read and cleared by the query
+    gave_up = int(bad[::32, ::256].sum())
+    assert p.faults() == gave_up
+    assert p.faults() == 0
+    if gave_up == 0:
+        pytest.skip("every wavefront found its row block complete at the first look (nothing gave up)")
+    # a limit that is not a whole number in range is refused, not read as 0
+    for garbage in ("-1", "many", "12x", "99999999999"):
+        monkeypatch.setenv("GERN_QK_SPIN_LIMIT", garbage)
+        with pytest.raises(gpu.GernError, match="GERN_QK_SPIN_LIMIT"):
+            p(dq, dk, S, scale)
     monkeypatch.delenv("GERN_QK_SPIN_LIMIT")
     p(dq, dk, S, scale)
     torch.cuda.synchronize()
     got = S.cpu().numpy()
     assert np.max(np.abs(got - want) / want) < 1e-2
+    assert p.faults() == 0
+
+
+def test_qk_softmax_tile_kernel_reports_logits_that_do_not_fit(gpu, oracle):
+    # A row statistic travels as a sixteen-bit shift: logits beyond 32767 in log2 units (or not a number)
+    # cannot be exchanged, their rows come back NaN, and the pipeline counts the (row, block of 256 keys)
+    # pairs; rows that fit are untouched.
+    import torch
+    M, N, D = 64, 512, 64
+    q = oracle.normal((M, D), 91)
+    k = oracle.normal((N, D), 92)
+    q[5, :] = 256.0          # row 5 against key 7: 64 * 256 * 256 * scale, far beyond the range
+    k[7, :] = 256.0
+    k[300, 3] = np.nan       # one key that poisons every row's second block of 256 keys
+    qb, _ = oracle.to_bf16(q)
+    kb, _ = oracle.to_bf16(k)
+    p = gpu.QKSoftmax(D, N)
+    S = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, np.float32(1.0))
+    torch.cuda.synchronize()
+    got = S.cpu().numpy()
+    assert np.all(np.isnan(got))  # the NaN key reaches every row's sum
+    assert p.faults() == M + 1    # every row's second block, and row 5's first
+    assert p.faults() == 0
+    kb[300, 3] = 0
+    p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, np.float32(1.0))
+    torch.cuda.synchronize()
+    got = S.cpu().numpy()
+    assert np.all(np.isnan(got[5])) and not np.any(np.isnan(np.delete(got, 5, axis=0)))
+    assert p.faults() == 1
 
 
 def test_qk_softmax_full_size(gpu, oracle):

@@ -242,3 +242,31 @@ def test_division_by_powers_of_two_is_exact(oracle):
     for d in (2.0, 4.0, 8.0):
         for lo, hi in ((0, 1 << 24), (0x3F000000, 0x3F000000 + (1 << 22)), (0x80000000, 0x80000000 + (1 << 24))):
             assert oracle.lib().oracle_quotient_mismatches(d, lo, hi, None, None, None) == 0
+
+
+def test_max_ulp_known_answers(oracle):
+    """max_ulp is the yardstick of the blur parity tests: known distances, so that `== 0` there means
+    bit-equal apart from the sign of zero (which those tests compare separately)."""
+    one = np.float32(1.0)
+    up = np.nextafter(one, np.float32(2.0))
+    assert oracle.max_ulp([one], [one]) == 0
+    assert oracle.max_ulp([one], [up]) == 1 and oracle.max_ulp([up], [one]) == 1
+    three = np.array([0x3F800003], dtype=np.uint32).view(np.float32)
+    assert oracle.max_ulp([one], three) == 3
+    # the worst element wins, wherever it sits
+    a = np.full(1000, 0.375, dtype=np.float32)
+    b = a.copy()
+    b[617] = np.nextafter(np.nextafter(b[617], np.float32(1.0)), np.float32(1.0))
+    assert oracle.max_ulp(a, b) == 2
+    # across a binade boundary and across zero the distance counts representable numbers
+    below_two = np.nextafter(np.float32(2.0), np.float32(0.0))
+    assert oracle.max_ulp([below_two], [np.nextafter(np.float32(2.0), np.float32(3.0))]) == 2
+    tiny = np.array([1], dtype=np.uint32).view(np.float32)  # the smallest subnormal
+    assert oracle.max_ulp(tiny, -tiny) == 2
+    assert oracle.max_ulp([np.float32(0.0)], [np.float32(-0.0)]) == 0  # documented: the sign of zero is not a distance
+    # a NaN on either side is never "close"
+    assert oracle.max_ulp([np.float32(np.nan)], [one]) == 0xFFFFFFFF
+    assert oracle.max_ulp([one], [np.float32(np.nan)]) == 0xFFFFFFFF
+    assert oracle.max_ulp([one, np.float32(np.nan)], [one, np.float32(np.nan)]) == 0xFFFFFFFF
+    # far apart: one against minus one
+    assert oracle.max_ulp([one], [-one]) == 2 * 0x3F800000
