@@ -116,3 +116,22 @@ __global__ void __launch_bounds__(64 * gernels::qk_waves(N)) check_qk_softmax(ge
 }
 template __global__ void check_qk_softmax<4096, 128>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32, float);
 template __global__ void check_qk_softmax<1024, 64>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32, float);
+
+#include "gernels/qk_tiles.h"
+
+// The tile program of the fused QK^T softmax: one workgroup per 256 x 256 tile of S.
+template<int64_t D>
+__global__ void __launch_bounds__(512) check_qk_softmax_tiles(gernels::MatrixBF16 Q, gernels::MatrixBF16 K, gernels::MatrixF32 S,
+                                                             gernels::RowStatsExchange exchange, float scale) {
+    const int64_t x = (int64_t)blockIdx.y * 256, y = (int64_t)blockIdx.x * 256;
+    auto session = exchange.open();
+    auto out = S.template view_score_tile<256, 256>(x, y);
+    auto logits = gernels::allocate_score_tile<256, 256>();
+    auto q = Q.template view<256, D>(x, 0);
+    auto k = K.template view<256, D>(y, 0);
+    gernels::qk_scaled(q, k, logits, scale);
+    gernels::softmax_rows_across_tiles(logits, session, out);
+    S.store_score_tile(x, y, out);
+}
+template __global__ void check_qk_softmax_tiles<128>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32, gernels::RowStatsExchange, float);
+template __global__ void check_qk_softmax_tiles<192>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32, gernels::RowStatsExchange, float);

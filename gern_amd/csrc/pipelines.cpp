@@ -16,6 +16,7 @@
 
 #include <cerrno>
 #include <cmath>
+#include <cstdio>
 #include <cstring>
 #include <algorithm>
 #include <cstdlib>
@@ -779,7 +780,7 @@ int gern_gemm_schedule_create(int schedule, int flags, gern_pipeline *out) {
             }
         };
         AbstractDataTypePtr A, B;
-        AbstractDataTypePtr C(schedule == 10 ? static_cast<const AbstractDataType *>(new const CWrittenBack("C", false))
+        AbstractDataTypePtr C(schedule != 3 ? static_cast<const AbstractDataType *>(new const CWrittenBack("C", false))
                                              : static_cast<const AbstractDataType *>(new const CType("C", false)));
         if (schedule == 3) {
             A = AbstractDataTypePtr(new const annot::MatrixGlobalToShared<N, N>("A", false));
@@ -800,27 +801,65 @@ int gern_gemm_schedule_create(int schedule, int flags, gern_pipeline *out) {
         auto &mm_sp = mm[{{"k_dim", k_dim}}];
         Composable program;
         if (schedule == 10) {
-            // kernel_10.cu:108-131: block tile -> wavefront tile -> one output per lane, register copies of C, A and B
+            // kernel_10.cu:108-131: block tile -> wavefront tile -> one output per lane, register copies of C, A and B.
+            // K tiles of 32: a lane then holds 32 + 32 operand values, within the 128 registers that a
+            // workgroup of 1024 threads leaves each lane (64-deep tiles spill to scratch memory).
+            int64_t kt10 = 32;
+            if (const char *v = std::getenv("GERN_SCHEDULE_TILES"); v != nullptr && experiments()) {
+                kt10 = std::atoll(v);
+            }
             Composable per_lane = Stage(
                 C, in_registers.getQueryFunction(), in_registers.getInsertFunction(),
                 Stage(A, in_registers.getQueryFunction(),
                       Stage(B, in_registers.getQueryFunction(),
                             Reduce(k_dim, thread_k.bind(8))(Stage(A, view_of.getView(), Stage(B, view_of.getView(), mm_sp(A, B, C)))))));
-            Composable lanes = (Tile(C["row"], thread_x.bind(1)) || Grid::Unit::THREAD_X_IN_WRAPS)(
-                (Tile(C["col"], thread_y.bind(1)) || Grid::Unit::THREAD_Y_IN_WRAPS)(per_lane));
-            Composable waves =
-                (Tile(C["row"], warp_x.bind(64)) || Grid::Unit::WARP_Y)((Tile(C["col"], warp_y.bind(16)) || Grid::Unit::WARP_X)(lanes));
-            program = Global((Tile(C["row"], block_x.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(16)) || Grid::Unit::BLOCK_Y)(
-                                 Reduce(k_dim, k_tiled.bind(64))(Stage(A, Stage(B, waves))))),
-                             {{Grid::Dim::BLOCK_DIM_Y, lanes_y.bind(16)}}, smem_size, annot::LdsManager(smem_size));
-        } else {
-            // kernel_3.cu:61-75 / kernel_6.cu:61-74: block tile staged through LDS, 4 x 4 outputs per thread;
-            // 64 x 64 block tiles make workgroups of 256 threads
-            Composable inner = Stage(A, schedule == 3 ? view_of.getView() : view_of.getViewVec(),
-                                     Stage(B, schedule == 3 ? view_of.getView() : view_of.getViewVec(), mm_sp(A, B, C)));
-            if (schedule == 3) {
-                inner = Reduce(k_dim, one_val.bind(16))(inner);
+            // The lanes of a wavefront (64 consecutive threadIdx.x) take 64 consecutive COLUMNS of one row of C:
+            // they then read the same element of the staged A tile (one LDS access, broadcast), consecutive
+            // elements of the staged B tile (all banks) and write consecutive floats of C.  kernel_10.cu puts
+            // consecutive lanes on consecutive rows; on the dense tiles that direct loads leave in LDS that makes
+            // every lane of a read hit the same bank (measured: 2064 us at 1024^3 against the time below).
+            const bool rows_on_lanes = std::getenv("GERN_SCHEDULE_ROWS_ON_LANES") != nullptr && experiments();
+            if (rows_on_lanes) {
+                Composable lanes = (Tile(C["row"], thread_x.bind(1)) || Grid::Unit::THREAD_X_IN_WRAPS)(
+                    (Tile(C["col"], thread_y.bind(1)) || Grid::Unit::THREAD_Y_IN_WRAPS)(per_lane));
+                Composable waves =
+                    (Tile(C["row"], warp_x.bind(64)) || Grid::Unit::WARP_Y)((Tile(C["col"], warp_y.bind(16)) || Grid::Unit::WARP_X)(lanes));
+                program = Global((Tile(C["row"], block_x.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(16)) || Grid::Unit::BLOCK_Y)(
+                                     Reduce(k_dim, k_tiled.bind(kt10))(Stage(A, Stage(B, waves))))),
+                                 {{Grid::Dim::BLOCK_DIM_Y, lanes_y.bind(16)}}, smem_size, annot::LdsManager(smem_size));
+            } else {
+                Composable lanes = (Tile(C["col"], thread_y.bind(1)) || Grid::Unit::THREAD_X_IN_WRAPS)(
+                    (Tile(C["row"], thread_x.bind(1)) || Grid::Unit::THREAD_Y_IN_WRAPS)(per_lane));
+                Composable waves =
+                    (Tile(C["col"], warp_y.bind(64)) || Grid::Unit::WARP_Y)((Tile(C["row"], warp_x.bind(16)) || Grid::Unit::WARP_X)(lanes));
+                program = Global((Tile(C["col"], block_y.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["row"], block_x.bind(16)) || Grid::Unit::BLOCK_Y)(
+                                     Reduce(k_dim, k_tiled.bind(kt10))(Stage(A, Stage(B, waves))))),
+                                 {{Grid::Dim::BLOCK_DIM_Y, lanes_y.bind(16)}}, smem_size, annot::LdsManager(smem_size));
             }
+        } else if (schedule == 6) {
+            // The composition of kernel_6.cu:61-74 (block tile staged through LDS 16 bytes per lane, thread
+            // tiles, windows of the staged tiles per thread) with one more Stage: the thread's tile of C is
+            // copied into registers.  That copy does not depend on the loop over K tiles, so the lowering
+            // makes it before the loop and writes it back after it, and matrix_multiply runs on a register
+            // tile (the reference's composition multiplies into C in global memory, a load and a store per
+            // term).  64 x 64 block tiles and 4 x 4 outputs per thread make workgroups of four wavefronts and
+            // 256 workgroups at 1024^2: one per compute unit.
+            int64_t bm = 64, bn = 64, kt = 64, tm = 4, tn = 4;
+            if (const char *v = std::getenv("GERN_SCHEDULE_TILES"); v != nullptr && experiments()) {
+                long long a[5] = {bm, bn, kt, tm, tn};
+                std::sscanf(v, "%lld,%lld,%lld,%lld,%lld", &a[0], &a[1], &a[2], &a[3], &a[4]);
+                bm = a[0], bn = a[1], kt = a[2], tm = a[3], tn = a[4];
+            }
+            Composable per_thread = Stage(C, in_registers.getQueryFunction(), in_registers.getInsertFunction(),
+                                          Stage(A, view_of.getViewVec(), Stage(B, view_of.getViewVec(), mm_sp(A, B, C))));
+            program = Global((Tile(C["row"], block_x.bind(bm)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(bn)) || Grid::Unit::BLOCK_Y)(
+                                 Reduce(k_dim, k_tiled.bind(kt))(Stage(A, Stage(B, (Tile(C["row"], thread_x.bind(tm)) || Grid::Unit::THREAD_Y)(
+                                                                                       (Tile(C["col"], thread_y.bind(tn)) || Grid::Unit::THREAD_X)(per_thread))))))),
+                             {}, smem_size, annot::LdsManager(smem_size));
+        } else {
+            // kernel_3.cu:61-75: block tile staged through LDS one float per lane, 4 x 4 outputs per thread multiplied
+            // straight into C in global memory; 64 x 64 block tiles make workgroups of 256 threads
+            Composable inner = Reduce(k_dim, one_val.bind(16))(Stage(A, view_of.getView(), Stage(B, view_of.getView(), mm_sp(A, B, C))));
             program = Global((Tile(C["row"], block_x.bind(64)) || Grid::Unit::BLOCK_X)((Tile(C["col"], block_y.bind(64)) || Grid::Unit::BLOCK_Y)(
                                  Reduce(k_dim, k_tiled.bind(16))(Stage(A, Stage(B, (Tile(C["row"], thread_x.bind(4)) || Grid::Unit::THREAD_Y)(
                                                                                        (Tile(C["col"], thread_y.bind(4)) || Grid::Unit::THREAD_X)(inner))))))),
@@ -846,6 +885,9 @@ int gern_gemm_schedule_run(gern_pipeline p, const float *A, const float *B, floa
     }
     hip::GlobalMatrixF32 a{const_cast<float *>(A)}, b{const_cast<float *>(B)}, c{C};
     int64_t smem = 48 * 1024;
+    if (const char *v = std::getenv("GERN_SCHEDULE_LDS_KB"); v != nullptr && experiments()) {
+        smem = std::atoll(v) * 1024;
+    }
     try {
         p->runner->setStream(stream);
         p->runner->evaluate({{"A", &a}, {"B", &b}, {"C", &c}, {"smem_size", &smem}});

@@ -16,7 +16,7 @@
 //    instruction), which fixes the LDS layout to the dense one;
 //  * LDS rows are padded by one 16-byte slot when their pitch would be a
 //    multiple of 128 bytes (every row on the same banks);
-//  * LDS comes from the free-list allocator in lds_alloc.h and is given back
+//  * LDS comes from the stack allocator in lds_alloc.h and is given back
 //    by free_smem().
 #pragma once
 
@@ -336,6 +336,54 @@ template<int64_t k_dim, typename AT, typename BT, typename CT>
 __device__ __forceinline__ void matrix_multiply(const AT &A, const BT &B, CT &C) {
     for (int64_t i = 0; i < AT::row; i++) {
         for (int64_t j = 0; j < BT::col; j++) {
+            for (int64_t k = 0; k < k_dim; k++) {
+                C(i, j) += A(i, k) * B(k, j);
+            }
+        }
+    }
+}
+
+// The same product, term by term in the same k order per element of C, for operands that are tiles (or
+// windows of tiles) in LDS and a tile of C in the thread's registers: four steps of k at a time, the thread
+// reads its H rows of A (16 bytes each) and the four rows of B (W consecutive floats each, 16 bytes at a
+// time) once and does 4 H W multiply-adds on them.  This is the overload a schedule reaches when it stages C
+// into registers (Stage(C, query_2_reg_no_vector, ...)) around operands staged into LDS; windows that are
+// not 16-byte aligned take the scalar loop.
+template<int64_t k_dim, int64_t HA, int64_t WA, int64_t LA, int64_t HB, int64_t WB, int64_t LB, int64_t H, int64_t W>
+__device__ __forceinline__ void matrix_multiply(const LdsTile<HA, WA, LA> &A, const LdsTile<HB, WB, LB> &B, RegTile<H, W> &C) {
+    static_assert(HA == H && WB == W && WA >= k_dim && HB >= k_dim, "tile shapes of C = A B");
+    constexpr bool vec = (k_dim % 4 == 0) && (W % 4 == 0) && (LA % 4 == 0) && (LB % 4 == 0);
+    if (vec && ((((uint64_t)A.data) | ((uint64_t)B.data)) & 15u) == 0) {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int64_t k = 0; k < (vec ? k_dim : 0); k += 4) {
+            f4 a[H], b[4][W / 4 > 0 ? W / 4 : 1];
+#pragma unroll
+            for (int64_t i = 0; i < H; i++) {
+                a[i] = *reinterpret_cast<const f4 *>(A.data + i * LA + k);
+            }
+#pragma unroll
+            for (int64_t kk = 0; kk < 4; kk++) {
+#pragma unroll
+                for (int64_t j = 0; j < W / 4; j++) {
+                    b[kk][j] = *reinterpret_cast<const f4 *>(B.data + (k + kk) * LB + 4 * j);
+                }
+            }
+#pragma unroll
+            for (int64_t kk = 0; kk < 4; kk++) {
+#pragma unroll
+                for (int64_t i = 0; i < H; i++) {
+#pragma unroll
+                    for (int64_t j = 0; j < W; j++) {
+                        C(i, j) += a[i][kk] * b[kk][j / 4][j % 4];
+                    }
+                }
+            }
+        }
+        return;
+    }
+    for (int64_t i = 0; i < H; i++) {
+        for (int64_t j = 0; j < W; j++) {
             for (int64_t k = 0; k < k_dim; k++) {
                 C(i, j) += A(i, k) * B(k, j);
             }

@@ -20,18 +20,21 @@
 // gernels (apps/common/impl/impl.h:7-188: max, subtract, exp, sum, divide) with
 // the two reductions finished across workgroups, as the reference's
 // grid_reduce_total finishes a sum across blocks with a device-scope atomic
-// (gernels/cccl/wrappers/reduce_wrappers.cuh:42-61).  The five stages are ONE
-// gernel here because they are pipelined over the two 16-row halves of a
-// wavefront's rows: the statistics of the first half are on their way to the
-// other workgroups while the exponentials of the second are computed, and the
-// first half is being stored while the second waits for its statistics (as
-// three gernels with one exchange for all rows: 25.1 us at 4096 x 4096 x 128;
-// this way 22.2 us, measured in one process).
+// (gernels/cccl/wrappers/reduce_wrappers.cuh:42-61).
 //
 // Eight wavefronts; wavefront w owns rows [32 w, 32 w + 32) of the tile and all
-// 256 columns, as 2 x 16 v_mfma_f32_16x16x32_bf16 tiles.  MFMA column j of
-// tile tn = 4 g + t stands for key 64 g + 4 j + t, so a lane holds four
-// consecutive columns of S per group g and stores them with one 16-byte store.
+// 256 columns, as eight v_mfma_f32_32x32x16_bf16 tiles that are computed
+// TRANSPOSED: the keys are the rows of the matrix instruction and the queries
+// its columns, so lane l holds, of query row 32 w + l % 32, the 128 scores of
+// keys 32 t + 8 a + 4 (l / 32) + b (tile t < 8, a < 4, b < 4).  A row of S is
+// thus spread over just two lanes (l and l + 32): its maximum and its sum are
+// 128 operations inside a lane and ONE exchange between the two, no DPP
+// butterflies, and the four scores b = 0 .. 3 are consecutive columns of S, one
+// 16-byte store.  (The 16 x 16 x 32 instruction, whose accumulators put a row
+// on sixteen lanes with four columns each, runs at HALF the rate on this GPU --
+// measured with loops of nothing but MFMAs: 1.23 against 2.46 PFLOP/s at
+// 2.4 GHz -- and the butterflies over sixteen lanes were a third of the
+// vector-ALU work of the softmax.)
 //
 // The exchange.  An entry is one 64-bit word per (row, column block): s in the
 // upper half, below it m as a sixteen-bit integer (a row is shifted by
@@ -47,21 +50,18 @@
 // another shape is never mistaken for a new one.  Entries are written and read
 // with agent-scope atomic accesses, which go to the memory side past the
 // caches that are private to an XCD; no cache is written back or invalidated.
-// Such reads run at about 3 TB/s over the whole GPU, and every tile reads the
-// entries of its whole row block, so the size of an entry is what the exchange
-// costs: 8 MiB and 2.5 us at 4096 x 4096 (entries of 16 bytes that held m as a
-// float: twice that).  Each wavefront polls the sixteen entries of its own 32
-// rows on its own.  Workgroup ids run along the columns, so the workgroups of
-// a row block are dispatched together; a workgroup waits only for workgroups
-// of its own row block, and those never wait for a later one.  The wait is
-// bounded all the same: after spin_limit polls a wavefront gives up and stores
-// NaN in its rows.  Logits beyond +-32767 in log2 units (22 000 in natural
-// units) do not fit an entry; their rows come out as NaN.  Neither goes
-// unnoticed by the host: state[2] counts the wavefronts that gave up and
-// state[3] the (row, column block) pairs whose shift did not fit or whose
-// logits were not all numbers, for the host to read and clear after the launch (the reference
-// checks for an error after every launch,
-// include/gern/codegen/helpers/check_last_error.h:7-18).
+// Each wavefront polls the sixteen entries of its own 32 rows on its own (lane
+// l the column blocks 8 (l / 32) .. + 7 of row l % 32).  Workgroup ids run
+// along the columns, so the workgroups of a row block are dispatched together;
+// a workgroup waits only for workgroups of its own row block, and those never
+// wait for a later one.  The wait is bounded all the same: after spin_limit
+// polls a wavefront gives up and stores NaN in its rows.  Logits beyond
+// +-32767 in log2 units (22 000 in natural units) do not fit an entry; their
+// rows come out as NaN.  Neither goes unnoticed by the host: state[2] counts
+// the wavefronts that gave up and state[3] the (row, column block) pairs whose
+// shift did not fit or whose logits were not all numbers, for the host to read
+// and clear after the launch (the reference checks for an error after every
+// launch, include/gern/codegen/helpers/check_last_error.h:7-18).
 //
 // Two launches that use the same exchange must not overlap in time.
 #pragma once
@@ -70,8 +70,6 @@
 #include "gernels/softmax.h"
 
 namespace gernels {
-
-typedef float score_f32x4_t __attribute__((ext_vector_type(4)));
 
 // Launch numbers run from 0 to kRowStatsTagPeriod - 1; a tag is the number + 1,
 // and 0 is a word that was never written.
@@ -111,29 +109,51 @@ struct RowStatsExchange {
     }
 };
 
+
 namespace detail {
 // Wavefronts of the workgroup that are done with the exchange.  qk_scaled clears
 // it ahead of its first barrier and softmax_rows_across_tiles counts in it, so
-// that the exchange needs no barrier of its own: the wavefronts of a workgroup
-// finish their exponentials up to a microsecond or two apart (a SIMD serves its older
-// wavefront first), and a wavefront exchanges only with its namesakes in the
-// other tiles of the row block, so the early ones are storing their rows while
-// the late ones still compute.
+// that the exchange needs no barrier of its own: a wavefront exchanges only with
+// its namesakes in the other tiles of the row block, and the wavefronts of a
+// workgroup reach the exchange a microsecond or two apart (a SIMD serves its
+// older wavefront first), so the early ones are storing their rows while the
+// late ones still compute.
 __shared__ unsigned int row_stats_waves_done;
+
+// The two LDS stages of qk_scaled (64 KiB each: 256 rows of Q, then 256 keys of K, 128 bytes per row).
+// Once every wavefront of the workgroup has read its last fragment (qk_waves_done_reading counts them),
+// softmax_rows_across_tiles turns its rows around through the first one on their way to memory.
+constexpr int kQkStageHalf = 256 * 128;  // bytes of one operand's stage
+__shared__ __attribute__((aligned(16))) unsigned char qk_stage_even[2 * kQkStageHalf];
+__shared__ __attribute__((aligned(16))) unsigned char qk_stage_odd[2 * kQkStageHalf];
+__shared__ unsigned int qk_waves_done_reading;
+
+// Where the entry of (row, column block) lies: the 256 rows of a row block side by side per column block, so
+// that the 32 lanes that publish or read one column block for 32 consecutive rows touch 256 consecutive
+// bytes (with the rows of a column block apart, every 8-byte entry was a memory access of its own, and a
+// round of polls over all tiles took microseconds).  `pitch` entries per row, at least the number of column blocks.
+__device__ __forceinline__ long long row_stats_entry(long long row, int block, int pitch) {
+    return ((row >> 8) * pitch + block) * 256 + (row & 255);
+}
+
+// The value that lane l ^ 32 holds (the other half of a row of scores).
+__device__ __forceinline__ float other_half(float x) {
+    return as_float(__builtin_amdgcn_ds_bpermute((lane_id() ^ 32) * 4, as_int(x)));
+}
 }  // namespace detail
 
-// A 256 x 256 tile of scores spread over eight wavefronts: acc[tm][4 g + t][i]
-// is row 32 w + 16 tm + 4 (lane / 16) + i, column 64 g + 4 (lane % 16) + t,
-// in units of `unit` (value = acc * unit) as qk_scaled leaves it, plain afterwards.
-// shift / sum: the statistics of the lane's eight rows over the tile's columns.
+// A 256 x 256 tile of scores spread over eight wavefronts: acc[t][4 a + b] of lane l
+// is row 32 w + l % 32, column 32 t + 8 a + 4 (l / 32) + b, in units of `unit`
+// (value = acc * unit) as qk_scaled leaves it, plain afterwards.
+// shift / sum: the statistics of the lane's row over the tile's columns.
 template<int64_t R, int64_t C>
 struct ScoreTile {
     static_assert(R == 256 && C == 256, "score tiles are 256 x 256");
     static constexpr int64_t rows = R;
     static constexpr int64_t cols = C;
-    score_f32x4_t acc[2][16];
-    float shift[2][4];
-    float sum[2][4];
+    f32x16_t acc[8];
+    float shift;
+    float sum;
     float unit;
     int valid_cols;  // columns of the tile that exist (keys)
     // A view of a matrix (view_score_tile): the matrix and where the tile's first
@@ -168,32 +188,65 @@ __device__ __forceinline__ ScoreTile<R, C> MatrixF32::view_score_tile(int64_t x,
 
 namespace detail {
 
-// Row 16 tm + i of each lane's rows (32 w + 4 (lane / 16) + that), every value
-// times f, 16 bytes per lane and store.
-template<int64_t R, int64_t C>
-__device__ __forceinline__ void store_score_row(const MatrixF32 &m, int64_t x, int64_t y, const ScoreTile<R, C> &t, int tm, int i, float f) {
+// The wavefront's 32 rows of the tile at (x, y) of m, every value times f.  A lane holds ONE row
+// (32 bytes of it per group of four accumulators, side by side with lane l ^ 32), so stored from the
+// registers as they are an instruction would write 32 bytes of each of 32 rows: measured, such stores take
+// three times as long as whole lines (36.5 against about 11 us for the 64 MiB of a 4096 x 4096 result).
+// Each 32 x 32 tile is therefore turned around through LDS: written as the lanes hold it (row l % 32,
+// 16-byte piece 2 a + l / 32 at position piece ^ ((row >> 1) & 7), which keeps both directions free of
+// bank conflicts), read back with eight lanes per row, and stored: an instruction then writes eight whole
+// 128-byte lines.  `lds` is 8 KiB that belong to this wavefront (two tiles: the next one is written while
+// the last one is read).
+template<int POLICY, int64_t R, int64_t C>
+__device__ __forceinline__ void store_score_rows(const MatrixF32 &m, int64_t x, int64_t y, const ScoreTile<R, C> &t, float f,
+                                                 unsigned char *lds) {
+    typedef float f32x4_native __attribute__((ext_vector_type(4)));
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
-    const int jl = lane % 16;
-    const int64_t rr = x + 32 * w + 16 * tm + 4 * (lane / 16) + i;
-    if (rr >= m.row) {
-        return;
-    }
-    float *p = m.data + rr * m.lda;
+    const int n = lane % 32, h = lane / 32;
+    const int put = n * 128, put_swz = (n >> 1) & 7;
+    const int64_t span = (m.row - 1) * m.lda + m.col;
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const int64_t cc = y + 64 * g + 4 * jl;
-        const float4 val = make_float4(t.acc[tm][4 * g + 0][i] * f, t.acc[tm][4 * g + 1][i] * f, t.acc[tm][4 * g + 2][i] * f,
-                                       t.acc[tm][4 * g + 3][i] * f);
-        if (cc + 3 < m.col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
-            store_result16<kThroughStores>(m.data, (m.row - 1) * m.lda + m.col, rr * m.lda + cc, val);
-        } else {
-            if (cc + 0 < m.col) p[cc + 0] = val.x;
-            if (cc + 1 < m.col) p[cc + 1] = val.y;
-            if (cc + 2 < m.col) p[cc + 2] = val.z;
-            if (cc + 3 < m.col) p[cc + 3] = val.w;
+    for (int tn = 0; tn < 8; tn++) {
+        unsigned char *tile = lds + (tn & 1) * 4096;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const f32x4_native val = {t.acc[tn][4 * a + 0] * f, t.acc[tn][4 * a + 1] * f, t.acc[tn][4 * a + 2] * f, t.acc[tn][4 * a + 3] * f};
+            *reinterpret_cast<f32x4_native *>(tile + put + (((2 * a + h) ^ put_swz) * 16)) = val;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int r = 8 * j + lane / 8, piece = lane % 8;
+            const f32x4_native q = *reinterpret_cast<const f32x4_native *>(tile + r * 128 + ((piece ^ ((r >> 1) & 7)) * 16));
+            const int64_t rr = x + 32 * w + r, cc = y + 32 * tn + 4 * piece;
+            if (rr >= m.row) {
+                continue;
+            }
+            float *p = m.data + rr * m.lda;
+            const float4 val = make_float4(q[0], q[1], q[2], q[3]);
+            if (cc + 3 < m.col && ((((uint64_t)(p + cc)) & 15u) == 0)) {
+                store_result16<POLICY>(m.data, span, rr * m.lda + cc, val);
+            } else {
+                if (cc + 0 < m.col) p[cc + 0] = val.x;
+                if (cc + 1 < m.col) p[cc + 1] = val.y;
+                if (cc + 2 < m.col) p[cc + 2] = val.z;
+                if (cc + 3 < m.col) p[cc + 3] = val.w;
+            }
         }
     }
+}
+
+// The 8 KiB of the first stage that wavefront w may use once no wavefront reads the stages any more; waits
+// for that (normally it has long been so: the products end microseconds before the first row is final).
+__device__ __forceinline__ unsigned char *own_lds_after_products() {
+    const unsigned int waves = blockDim.x / kWaveSize;
+    while (__hip_atomic_load(&qk_waves_done_reading, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < waves) {
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return qk_stage_even + (threadIdx.x / kWaveSize) * 8192;
 }
 
 }  // namespace detail
@@ -203,13 +256,7 @@ __device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y
     if (t.stored) {  // its rows went out through the view
         return;
     }
-#pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            detail::store_score_row(*this, x, y, t, tm, i, 1.0f);
-        }
-    }
+    detail::store_score_rows<kThroughStores>(*this, x, y, t, 1.0f, detail::own_lds_after_products());
 }
 
 // The raw products Q K^T of the tile; S.unit = scale * log2(e).
@@ -218,9 +265,12 @@ __device__ __forceinline__ void MatrixF32::store_score_tile(int64_t x, int64_t y
 // round trip) in stages of 64 along the head dimension, two stages in flight
 // from the start: a stage is 256 rows of Q and 256 keys of K, 128 bytes each,
 // with the 16-byte piece c of LDS row r at position c ^ ((r >> 1) & 7), which
-// spreads the sixteen rows of one fragment read over all banks.  LDS row
-// 64 g + 16 t + j of the K stage holds key 64 g + 4 j + t: the sixteen keys of
-// MFMA tile 4 g + t are then sixteen consecutive LDS rows, like the rows of Q.
+// spreads the sixteen rows of one pass of a fragment read over all banks.
+// The loads (128 KiB per workgroup, 32 MiB out of L2 over all of them at
+// 4096 x 4096 x 128) are what this gernel waits for: its products end about
+// 4 us after the launch with either matrix instruction.  Stages of 32 (whose
+// products could start earlier) fetch half a cache line per row and
+// instruction and end a microsecond LATER.
 // Rows of Q and keys past the end of the matrices are read from the last
 // valid one (rows past the end are never stored, keys past the end are left
 // out of the statistics by softmax_rows_across_tiles).
@@ -229,26 +279,30 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
                                           ScoreTile<R, C> &S, float scale) {
     static_assert(D % 64 == 0 && D >= 64, "score tiles stage the head dimension in steps of 64");
     constexpr int NK = (int)(D / 64);
-    constexpr int HALF = 256 * 128;  // bytes of one operand's stage
-    __shared__ __attribute__((aligned(16))) unsigned char qk_stage_even[2 * HALF];
-    __shared__ __attribute__((aligned(16))) unsigned char qk_stage_odd[2 * HALF];
+    constexpr int HALF = detail::kQkStageHalf;
+    unsigned char *const qk_stage_even = detail::qk_stage_even;
+    unsigned char *const qk_stage_odd = detail::qk_stage_odd;
     const int lane = lane_id();
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
 
     S.unit = scale * 1.4426950408889634f;
     S.valid_cols = (int)K.rows;
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
+    for (int tn = 0; tn < 8; tn++) {
 #pragma unroll
-        for (int tn = 0; tn < 16; tn++) {
-            S.acc[tm][tn] = score_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < 16; i++) {
+            S.acc[tn][i] = 0.f;
         }
     }
     if (threadIdx.x == 0) {
         detail::row_stats_waves_done = 0u;  // seen by all after the first barrier below
+        detail::qk_waves_done_reading = 0u;
     }
     if (Q.rows <= 0 || K.rows <= 0) {  // workgroup-uniform
         __syncthreads();
+        if (lane == 0) {
+            __hip_atomic_fetch_add(&detail::qk_waves_done_reading, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
         return;
     }
     // Wavefront w issues Q instructions 4w .. 4w+3 and K instructions 4w .. 4w+3
@@ -263,12 +317,11 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
     int off_q[4], off_k[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const int r = 8 * (w * 4 + j) + lane / 8;  // LDS row
+        const int r = 8 * (w * 4 + j) + lane / 8;  // LDS row = row of Q, key of K
         const int piece = (lane % 8) ^ ((r >> 1) & 7);
         const int q_row = r < (int)Q.rows - 1 ? r : (int)Q.rows - 1;
         off_q[j] = (q_row * (int)Q.lda + piece * 8) * 2;
-        int key = 64 * (r / 64) + 4 * (r % 16) + (r / 16) % 4;
-        key = key < (int)K.rows - 1 ? key : (int)K.rows - 1;
+        const int key = r < (int)K.rows - 1 ? r : (int)K.rows - 1;
         off_k[j] = (key * (int)K.lda + piece * 8) * 2;
     }
     auto issue = [&](int kt, unsigned char *dst) {
@@ -283,24 +336,24 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
                                                      16, off_k[j], kt * 128, 0, 0);
         }
     };
-    // Fragments: lane l holds row / key l % 16 of an MFMA tile and the eight
-    // values 8 (l / 16) .. + 7 of a 32-deep step.  Every LDS address is one
-    // offset from its stage array (the compiler then orders reads of one stage
-    // against the loads into that stage only).
-    const int swz = ((lane % 16) >> 1) & 7;
-    const int a_off = (32 * w + (lane % 16)) * 128;
-    const int b_off = HALF + (lane % 16) * 128;
+    // Fragments of a 16-deep step: lane l holds row l % 32 (a key of a K tile,
+    // a query of this wavefront's rows of Q) and the eight values
+    // 8 (l / 32) .. + 7 of the step.  Every LDS address is one offset from its
+    // stage array (the compiler then orders reads of one stage against the
+    // loads into that stage only).
+    const int swz = ((lane % 32) >> 1) & 7;  // rows 32 t + l % 32: the other terms are multiples of 16
+    const int q_off = (32 * w + (lane % 32)) * 128;
+    const int k_off = HALF + (lane % 32) * 128;
     auto compute = [&](const unsigned char *stage) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            const int pos = ((4 * s + lane / 16) ^ swz) * 16;
-            const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(stage + (a_off + pos));
-            const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(stage + (a_off + 16 * 128 + pos));
+        for (int s = 0; s < 4; s++) {
+            const int pos = ((2 * s + lane / 32) ^ swz) * 16;
+            const bf16x8_t q = *reinterpret_cast<const bf16x8_t *>(stage + (q_off + pos));
 #pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                const bf16x8_t b = *reinterpret_cast<const bf16x8_t *>(stage + (b_off + tn * 16 * 128 + pos));
-                S.acc[0][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, S.acc[0][tn], 0, 0, 0);
-                S.acc[1][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, S.acc[1][tn], 0, 0, 0);
+            for (int tn = 0; tn < 8; tn++) {
+                const bf16x8_t k = *reinterpret_cast<const bf16x8_t *>(stage + (k_off + tn * 32 * 128 + pos));
+                // keys are the rows of the product, queries its columns
+                S.acc[tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k, q, S.acc[tn], 0, 0, 0);
             }
         }
     };
@@ -325,6 +378,11 @@ __device__ __forceinline__ void qk_scaled(const GlobalView<R, D, uint16_t, false
             __builtin_amdgcn_s_barrier();
             issue(kt + 2, (kt & 1) ? qk_stage_odd : qk_stage_even);
         }
+    }
+    // this wavefront reads the stages no more
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    if (lane == 0) {
+        __hip_atomic_fetch_add(&detail::qk_waves_done_reading, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
 }
 
@@ -372,189 +430,161 @@ __device__ __forceinline__ void close_row_stats(const RowStatsSession &ex, unsig
 
 // out = softmax over the WHOLE rows of S that the tile `in` of scaled products
 // (value = acc * in.unit, in log2 units) is a 256-column piece of; `out` is a
-// view of S and its rows are stored through it.  Per 16-row half of a
-// wavefront's rows, in this order:
+// view of S and its rows are stored through it.  Per wavefront (32 rows, one
+// per pair of lanes):
 //
-//   half 0: m = floor(max), e = 2^(x - m), s = sum e; publish (m, s) per row
-//   half 1: the same
-//   half 0: wait for the sixteen column blocks' (m, s) of its rows, combine to
-//           (M, S), store e * 2^(m - M) / S
-//   half 1: the same
+//   m = floor(max), e = 2^(x - m), s = sum e; publish (m, s) per row
+//   wait for the sixteen column blocks' (m, s) of the rows, combine to (M, S)
+//   store e * 2^(m - M) / S
 //
-// so the entries of half 0 travel while half 1 is computed, and half 0 is
-// stored while half 1 waits.  An entry is published by lanes j < 4 of each
-// 16-lane row (row slot i = j of the half).
+// The two wavefronts of a SIMD do not run side by side: the SIMD serves the
+// older one first, so one is at its exponentials while the other multiplies,
+// and one waits for the exchange or stores while the other is at its
+// exponentials.
 template<int64_t R, int64_t C>
 __device__ __forceinline__ void softmax_rows_across_tiles(const ScoreTile<R, C> &in, const RowStatsSession &ex, ScoreTile<R, C> &out) {
     typedef unsigned long long u64;
-    // Rows per lane and pipeline step (slot r = 4 tm + i is row 16 tm + i of the lane's eight rows).  Measured
-    // at 4096 x 4096 x 128 in one process: 8 (one exchange for all rows) 24.3 us, 4 (the two halves) 21.7 us,
-    // 1 (row by row) 23.6 us.
-    constexpr int G = 4;
-    static_assert(G == 1 || G == 2 || G == 4 || G == 8, "group size");
     const int lane = lane_id();
     const int w = (int)(threadIdx.x / kWaveSize);
-    const int jl = lane % 16;
+    const int half = lane / 32;
     const float unit = in.unit;
     const bool partial = in.valid_cols < (int)C;  // workgroup-uniform: the last column block only
     const bool flip = unit < 0.f;                 // a negative scale turns the largest product into the smallest logit
     const int bj = out.col0 / (int)C, nbj = (int)gridDim.x;  // one workgroup per column block along x
-    const int64_t row0 = (int64_t)out.row0 + 32 * w + 4 * (lane / 16);
+    const int64_t row = (int64_t)out.row0 + 32 * w + lane % 32;
     const u64 tag = ex.tag;
     out.unit = 1.0f;
     out.valid_cols = in.valid_cols;
-    unsigned int unfit = 0;  // rows of this lane whose shift does not fit an entry (the same in all sixteen lanes of a row)
+
+    // ---- the tile's own statistics of the row ----
 #pragma unroll
-    for (int grp = 0; grp < 8 / G; grp++) {
+    for (int tn = 0; tn < 8; tn++) {
+        out.acc[tn] = in.acc[tn];
+    }
+    if (flip) {  // uniform
 #pragma unroll
-        for (int r = grp * G; r < grp * G + G; r++) {
-            const int tm = r / 4, i = r % 4;
-            float x[16];
-#pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                x[tn] = in.acc[tm][tn][i];
-            }
-            if (flip) {
-#pragma unroll
-                for (int tn = 0; tn < 16; tn++) {
-                    x[tn] = -x[tn];
-                }
-            }
-            if (partial) {
-#pragma unroll
-                for (int tn = 0; tn < 16; tn++) {
-                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
-                    x[tn] = key < in.valid_cols ? x[tn] : -__builtin_huge_valf();
-                }
-            }
-            float m = x[0];
-#pragma unroll
-            for (int tn = 1; tn < 16; tn++) {
-                m = __builtin_fmaxf(m, x[tn]);
-            }
-            m = __builtin_fmaxf(m, dpp_move<0xB1>(m));
-            m = __builtin_fmaxf(m, dpp_move<0x4E>(m));
-            m = __builtin_fmaxf(m, dpp_move<0x141>(m));
-            m = __builtin_fmaxf(m, dpp_move<0x140>(m));
-            const float a = flip ? -unit : unit;
-            // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
-            // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
-            const float whole = __builtin_floorf(m * a);
-            const float shift = __builtin_fminf(__builtin_fmaxf(whole, -32768.0f), 32767.0f);
-            float s = 0.f;
-#pragma unroll
-            for (int tn = 0; tn < 16; tn++) {
-                // a masked column is -inf: 2^-inf = 0 unless a == 0 (0 * inf), which the test below catches
-                float e = __builtin_amdgcn_exp2f(__builtin_fmaf(x[tn], a, -shift));
-                if (partial) {
-                    const int key = 64 * (tn / 4) + 4 * jl + (tn % 4);
-                    e = key < in.valid_cols ? e : 0.f;
-                }
-                out.acc[tm][tn][i] = e;
-                s += e;
-            }
-            s += dpp_move<0xB1>(s);
-            s += dpp_move<0x4E>(s);
-            s += dpp_move<0x141>(s);
-            s += dpp_move<0x140>(s);
-            out.shift[tm][i] = shift;
-            out.sum[tm][i] = s;
-            // the largest logit beyond an entry's range or not a number, or a logit that is not a number
-            unfit += (whole != shift || s != s) ? 1u : 0u;
+        for (int tn = 0; tn < 8; tn++) {
+            out.acc[tn] = -out.acc[tn];
         }
-        {
-            // lane j < G of each 16-lane row publishes slot grp * G + j
-            float m = out.shift[(grp * G) / 4][(grp * G) % 4], s = out.sum[(grp * G) / 4][(grp * G) % 4];
+    }
+    if (partial) {  // uniform
 #pragma unroll
-            for (int q = 1; q < G; q++) {
-                m = jl == q ? out.shift[(grp * G + q) / 4][(grp * G + q) % 4] : m;
-                s = jl == q ? out.sum[(grp * G + q) / 4][(grp * G + q) % 4] : s;
-            }
-            if (jl < G) {
-                const int r = grp * G + jl;
-                u64 *e = ex.entries + ((row0 + 16 * (r / 4) + (r % 4)) * ex.pitch + bj);
-                const u64 word = ((u64)(unsigned int)as_int(s) << 32) | ((u64)((unsigned int)(int)m & 0xFFFFu) << 16) | tag;
-                __hip_atomic_store(e, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int tn = 0; tn < 8; tn++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int key = 32 * tn + 8 * (i / 4) + 4 * half + (i % 4);
+                out.acc[tn][i] = key < in.valid_cols ? out.acc[tn][i] : -__builtin_huge_valf();
             }
         }
     }
-    if (unfit != 0u && jl == 0) {  // never, for logits that fit: one lane per 16-lane row reports its rows
-        __hip_atomic_fetch_add(ex.state + 3, unfit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    bool gave_up = false;
+    float m4[4] = {-__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf(), -__builtin_huge_valf()};
 #pragma unroll
-    for (int grp = 0; grp < 8 / G; grp++) {
-        // Lane j collects column block j (j + 16, ...) for the G rows it holds of this group.
-        float big_m[G], big_s[G];
+    for (int tn = 0; tn < 8; tn++) {
 #pragma unroll
-        for (int q = 0; q < G; q++) {
-            big_m[q] = -__builtin_huge_valf();
-            big_s[q] = 0.f;
+        for (int i = 0; i < 16; i++) {
+            m4[i % 4] = __builtin_fmaxf(m4[i % 4], out.acc[tn][i]);
         }
-        bool failed = false;
-        for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
-            const int b = b0 + jl;
-            u64 got[G];
-            int spins = 0;
-            for (;;) {
-                bool mine = true;
+    }
+    float m = __builtin_fmaxf(__builtin_fmaxf(m4[0], m4[1]), __builtin_fmaxf(m4[2], m4[3]));
+    m = __builtin_fmaxf(m, detail::other_half(m));
+    const float a = flip ? -unit : unit;
+    // The floor of the row's largest logit in log2 units (a >= 0), within what an entry of
+    // the exchange holds: the largest e is then in [1, 2) and no e that matters underflows.
+    const float whole = __builtin_floorf(m * a);
+    const float shift = __builtin_fminf(__builtin_fmaxf(whole, -32768.0f), 32767.0f);
+    // a masked column is -inf: 2^-inf = 0 unless a == 0 (0 * inf = NaN), which the masking after the loop catches
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tn = 0; tn < 8; tn++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            out.acc[tn][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(out.acc[tn][i], a, -shift));
+        }
+    }
+    if (partial) {  // uniform
+#pragma unroll
+        for (int tn = 0; tn < 8; tn++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int key = 32 * tn + 8 * (i / 4) + 4 * half + (i % 4);
+                out.acc[tn][i] = key < in.valid_cols ? out.acc[tn][i] : 0.f;
+            }
+        }
+    }
+#pragma unroll
+    for (int tn = 0; tn < 8; tn++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            s4[i % 4] += out.acc[tn][i];
+        }
+    }
+    float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    s += detail::other_half(s);
+    // The largest logit beyond an entry's range or not a number, or a logit that is not a number: the sum
+    // travels as NaN, which makes the whole row NaN in every tile.
+    const bool bad = whole != shift || s != s;
+    s = bad ? __builtin_nanf("") : s;
+    out.shift = shift;
+    out.sum = s;
+    if (half == 0) {
+        u64 *e = ex.entries + detail::row_stats_entry(row, bj, ex.pitch);
+        const u64 word = ((u64)(unsigned int)as_int(s) << 32) | ((u64)((unsigned int)(int)shift & 0xFFFFu) << 16) | tag;
+        __hip_atomic_store(e, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (bad && row < out.home.row) {  // never, for logits that fit (rows past the end repeat the last one)
+            __hip_atomic_fetch_add(ex.state + 3, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+
+    // ---- the statistics of the whole row: lane l collects column blocks 8 (l / 32) .. + 7 (+ 16, ...) ----
+    float big_m = -__builtin_huge_valf(), big_s = 0.f;
+    bool failed = false;
+    for (int b0 = 0; b0 < nbj; b0 += 16) {  // one pass for up to 4096 keys
+        u64 got[8];
+        int spins = 0;
+        for (;;) {
+            bool mine = true;
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const int b = b0 + 8 * half + q;
                 if (b < nbj) {
-#pragma unroll
-                    for (int q = 0; q < G; q++) {
-                        const int r = grp * G + q;
-                        const u64 *e = ex.entries + ((row0 + 16 * (r / 4) + (r % 4)) * ex.pitch + b);
-                        got[q] = __hip_atomic_load(e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-#pragma unroll
-                    for (int q = 0; q < G; q++) {
-                        mine = mine && (got[q] & 0xFFFFull) == tag;
-                    }
-                }
-                if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
-                    break;
-                }
-                if (++spins > ex.spin_limit) {  // wave-uniform
-                    failed = true;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(2);  // 0 to 32 measure the same
-            }
-            if (b < nbj) {
-#pragma unroll
-                for (int q = 0; q < G; q++) {
-                    const float m = (float)(short)(unsigned short)((got[q] >> 16) & 0xFFFFull), s = as_float((int)(unsigned int)(got[q] >> 32));
-                    const float top = __builtin_fmaxf(big_m[q], m);
-                    big_s[q] = big_s[q] * __builtin_amdgcn_exp2f(big_m[q] - top) + s * __builtin_amdgcn_exp2f(m - top);
-                    big_m[q] = top;
+                    got[q] = __hip_atomic_load(ex.entries + detail::row_stats_entry(row, b, ex.pitch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-        }
-        gave_up = gave_up || failed;
-        if (grp == 8 / G - 1) {
-            if (gave_up && lane == 0) {  // wave-uniform condition
-                __hip_atomic_fetch_add(ex.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                mine = mine && (b0 + 8 * half + q >= nbj || (got[q] & 0xFFFFull) == tag);
             }
-            detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
+            if (__builtin_amdgcn_ballot_w64(!mine) == 0) {
+                break;
+            }
+            if (++spins > ex.spin_limit) {  // wave-uniform
+                failed = true;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);  // 0 to 32 measure the same
         }
 #pragma unroll
-        for (int q = 0; q < G; q++) {
-            const int r = grp * G + q, tm = r / 4, i = r % 4;
-            const float m = big_m[q];
-            float top = m;
-            top = __builtin_fmaxf(top, dpp_move<0xB1>(top));
-            top = __builtin_fmaxf(top, dpp_move<0x4E>(top));
-            top = __builtin_fmaxf(top, dpp_move<0x141>(top));
-            top = __builtin_fmaxf(top, dpp_move<0x140>(top));
-            // a lane with no column block holds (-inf, 0) and adds 0 * 2^-inf = 0
-            float s = big_s[q] * __builtin_amdgcn_exp2f(m - top);
-            s += dpp_move<0xB1>(s);
-            s += dpp_move<0x4E>(s);
-            s += dpp_move<0x141>(s);
-            s += dpp_move<0x140>(s);
-            float f = __builtin_amdgcn_exp2f(out.shift[tm][i] - top) * (1.0f / s);
-            f = failed ? __builtin_nanf("") : f;
-            detail::store_score_row(out.home, out.row0, out.col0, out, tm, i, f);
+        for (int q = 0; q < 8; q++) {
+            if (b0 + 8 * half + q < nbj) {
+                const float em = (float)(short)(unsigned short)((got[q] >> 16) & 0xFFFFull), es = as_float((int)(unsigned int)(got[q] >> 32));
+                const float top = __builtin_fmaxf(big_m, em);
+                big_s = big_s * __builtin_amdgcn_exp2f(big_m - top) + es * __builtin_amdgcn_exp2f(em - top);
+                big_m = top;
+            }
         }
+    }
+    if (failed && lane == 0) {  // wave-uniform condition
+        __hip_atomic_fetch_add(ex.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    detail::close_row_stats(ex, &detail::row_stats_waves_done);  // this wavefront reads no entry from here on
+    {
+        // a lane with no column block holds (-inf, 0) and adds 0 * 2^-inf = 0
+        const float top = __builtin_fmaxf(big_m, detail::other_half(big_m));
+        float sum = big_s * __builtin_amdgcn_exp2f(big_m - top);
+        sum += detail::other_half(sum);
+        float f = __builtin_amdgcn_exp2f(shift - top) * (1.0f / sum);
+        f = failed ? __builtin_nanf("") : f;
+        detail::store_score_rows<kThroughStores>(out.home, out.row0, out.col0, out, f, detail::own_lds_after_products());
     }
     out.stored = true;
 }

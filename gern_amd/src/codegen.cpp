@@ -3,6 +3,7 @@
 #include "gern/codegen/codegen.h"
 
 #include <algorithm>
+#include <optional>
 #include <sstream>
 
 namespace gern {
@@ -374,6 +375,65 @@ public:
         }
     }
 
+    static constexpr int64_t kUnrollTrips = 32;
+    int loop_depth = 0;  // loops (not grid-mapped ranges) around the statement being emitted
+
+    // The value of an index expression when every variable in it is bound to a number.
+    static std::optional<int64_t> constantValue(const Expr &e) {
+        if (e.ptr == nullptr) {
+            return std::nullopt;
+        }
+        const ExprNode *n = e.ptr;
+        switch (n->kind) {
+        case ExprKind::Literal:
+            return static_cast<const LiteralNode *>(n)->i;
+        case ExprKind::Variable: {
+            const Variable v = to<Variable>(e);
+            return v.isBound() ? std::optional<int64_t>(v.getInt64Val()) : std::nullopt;
+        }
+        case ExprKind::ADTMember:
+        case ExprKind::GridDim:
+            return std::nullopt;
+        default:
+            break;
+        }
+        const auto *b = static_cast<const BinaryExprNode *>(n);
+        const auto x = constantValue(b->a), y = constantValue(b->b);
+        if (!x || !y) {
+            return std::nullopt;
+        }
+        switch (n->kind) {
+        case ExprKind::Add:
+            return *x + *y;
+        case ExprKind::Sub:
+            return *x - *y;
+        case ExprKind::Mul:
+            return *x * *y;
+        case ExprKind::Div:
+            return *y == 0 ? std::nullopt : std::optional<int64_t>(*x / *y);
+        case ExprKind::Mod:
+            return *y == 0 ? std::nullopt : std::optional<int64_t>(*x % *y);
+        default:
+            return std::nullopt;
+        }
+    }
+
+    // True if a loop (not a grid-mapped range) lies anywhere below n.
+    static bool containsLoop(const NodePtr &n) {
+        if (!n) {
+            return false;
+        }
+        if (n->kind == NodeKind::Interval) {
+            return !n->isMappedToGrid() || containsLoop(n->body);
+        }
+        for (const auto &c : n->children) {
+            if (containsLoop(c)) {
+                return true;
+            }
+        }
+        return false;
+    }
+
     void emitInterval(const NodePtr &n, int indent) {
         const Variable index = n->intervalVariable();
         const Expr extent = n->end - n->start.getB();
@@ -382,10 +442,20 @@ public:
         if (!n->isMappedToGrid()) {
             declared_vars.insert(index.getName());
             std::string i = index.getName();
+            // An innermost loop of a few steps, inside another loop, whose bounds are all bound at generation
+            // time is unrolled: per-thread register tiles indexed by the loop variable (RegTile::get_view) then
+            // have constant indices; indexed by a variable they live in scratch memory.  (The outermost loop
+            // of a kernel is the one that stages tiles and meets at barriers: that one stays a loop.)
+            const auto trips = constantValue(ceil);
+            if (loop_depth > 0 && trips && *trips > 1 && *trips <= kUnrollTrips && !containsLoop(n->body)) {
+                line(indent, "#pragma unroll");
+            }
+            loop_depth++;
             line(indent, "for (int64_t " + i + " = " + gen(n->start.getB()) + "; " + i + " < " + gen(n->end) + "; " +
                              i + " = " + i + " + " + gen(n->step) + ") {");
             emit(n->body, indent + 1);
             line(indent, "}");
+            loop_depth--;
             return;
         }
 

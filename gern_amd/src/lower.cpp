@@ -586,8 +586,19 @@ private:
             const std::string child = n->child.getName();
             adt_depth[child] = depthOf(by);
             auto &level = at_depth[adt_depth[child]];
+            // A data structure that a statement of this scope defines (allocates, computes or queries) is not
+            // a parameter of the kernel: a query of it must stay behind that statement.
+            const std::string parent = n->method.data.getName();
+            bool parent_is_parameter = true;
+            for (const auto &earlier : level) {
+                if ((earlier->kind == NodeKind::Allocate && earlier->call.output.getADTPtr().getName() == parent) ||
+                    (earlier->kind == NodeKind::Compute && earlier->adt.getName() == parent) ||
+                    (earlier->kind == NodeKind::Query && earlier->child.getName() == parent)) {
+                    parent_is_parameter = false;
+                }
+            }
             if (adt_depth[child] == 0 && n->method.call.args.empty() && n->method.call.template_args.empty() &&
-                !n->insert) {
+                !n->insert && parent_is_parameter) {
                 // A query that takes nothing (it opens a session on a parameter: a
                 // load whose result is needed much later) goes first, behind the
                 // launch declarations, so that its latency hides behind what follows.

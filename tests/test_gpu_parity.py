@@ -653,17 +653,28 @@ def test_qk_softmax_tile_kernel_launch_number_wraps_around(gpu, oracle, monkeypa
         p(_dev(small[0].view(np.int16)), _dev(small[1].view(np.int16)), S, scale, no_alloc=True)
 
 
-def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, monkeypatch):
+# The second shape splits a row block over two rounds of dispatch: 30 row blocks of 10 tiles are 300
+# workgroups on 256 compute units, so six tiles of the 26th row block start with the launch and its other four
+# only when a compute unit is free again.  With the normal limit the six wait for the four; with no polls
+# allowed they are certain to give up.
+@pytest.mark.parametrize("M,N,must_give_up", [(1024, 4096, False), (7680, 2560, True)])
+def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, monkeypatch, M, N, must_give_up):
     # With no polls allowed, a wavefront that does not find the statistics of
     # the whole row block at its first look gives up and stores NaN in its
     # rows: the launch still finishes, every row is either right or NaN, and
     # the next launch (with the normal limit) is right everywhere.
     import torch
-    M, N, D = 1024, 4096, 128
-    qb, _ = oracle.to_bf16(oracle.normal((M, D), 5))
-    kb, _ = oracle.to_bf16(oracle.normal((N, D), 6))
+    D = 128
+    qb, qv = oracle.to_bf16(oracle.normal((M, D), 5))
+    kb, kv = oracle.to_bf16(oracle.normal((N, D), 6))
     scale = np.float32(1.0 / np.sqrt(D))
-    want = oracle.qk_softmax(qb, kb, scale)
+    if M <= 1024:
+        want = oracle.qk_softmax(qb, kb, scale)
+    else:  # fp64 of the same bf16 values (the kernel is within 1e-5 of it, the oracle within 1e-2)
+        logits = (qv.astype(np.float64) @ kv.T.astype(np.float64)) * float(scale)
+        e = np.exp(logits - logits.max(axis=1, keepdims=True))
+        want = (e / e.sum(axis=1, keepdims=True)).astype(np.float32)
+        del logits, e
     p = gpu.QKSoftmax(D, 4096)
     dq, dk = _dev(qb.view(np.int16)), _dev(kb.view(np.int16))
     S = torch.zeros((M, N), dtype=torch.float32, device="cuda")
@@ -680,8 +691,7 @@ def test_qk_softmax_tile_kernel_gives_up_waiting_without_hanging(gpu, oracle, mo
     gave_up = int(bad[::32, ::256].sum())
     assert p.faults() == gave_up
     assert p.faults() == 0
-    if gave_up == 0:
-        pytest.skip("every wavefront found its row block complete at the first look (nothing gave up)")
+    assert gave_up > 0 or not must_give_up
     # a limit that is not a whole number in range is refused, not read as 0
     for garbage in ("-1", "many", "12x", "99999999999"):
         monkeypatch.setenv("GERN_QK_SPIN_LIMIT", garbage)
@@ -829,3 +839,67 @@ def test_destroying_pipelines_frees_their_code_objects(gpu, oracle):
         once()
     free_after, _ = torch.cuda.mem_get_info()
     assert free_before - free_after < 32 * 2 ** 20, (free_before, free_after)
+
+
+# ------------------------------------------------------------- LDS allocator ----
+def test_lds_allocator_is_a_stack_that_takes_releases_in_any_order(gpu):
+    # gernels/lds_alloc.h: blocks come from the top of a stack; a block released out of order gives its
+    # space back when the blocks above it are released too; requests that do not fit are counted.
+    import ctypes as C
+    import os
+    import torch
+    src = rb"""
+#include "gernels/lds_alloc.h"
+extern "C" __global__ void __launch_bounds__(256) lds_alloc_sequence(unsigned int *out, long long bytes) {
+    using namespace gernels;
+    lds_init(bytes);
+    unsigned char *base = gern_lds;
+    auto note = [&](int slot, unsigned int v) { if (threadIdx.x == 5) out[slot] = v; };
+    void *a = lds_alloc(1000);   // 1008 bytes after the 128-byte table
+    void *b = lds_alloc(64);
+    void *c = lds_alloc(16);
+    note(0, (unsigned int)((unsigned char *)a - base));
+    note(1, (unsigned int)((unsigned char *)b - base));
+    note(2, (unsigned int)((unsigned char *)c - base));
+    __syncthreads();
+    note(3, lds_in_use());
+    lds_free(b);                 // out of order: c is still above it
+    void *d = lds_alloc(32);     // goes above c, not into the hole
+    note(4, (unsigned int)((unsigned char *)d - base));
+    lds_free(d);
+    lds_free(c);                 // now b's hole is at the top too: the stack falls back to the end of a
+    void *e = lds_alloc(48);
+    note(5, (unsigned int)((unsigned char *)e - base));
+    lds_free(a);                 // a lies below e: stays until e goes
+    lds_free(e);
+    void *f = lds_alloc(4096);   // the whole heap again
+    note(6, (unsigned int)((unsigned char *)f - base));
+    note(7, lds_overflowed() ? 1u : 0u);
+    lds_free(f);
+    void *g = lds_alloc(bytes);  // cannot fit (the table takes 128 bytes): start of the heap, counted
+    note(8, (unsigned int)((unsigned char *)g - base));
+    __syncthreads();
+    note(9, lds_overflowed() ? 1u : 0u);
+    note(10, gern_lds_overflows);
+}
+"""
+    hip = gpu.hip_lib()
+    opts = (C.c_char_p * 1)(("-I" + os.path.dirname(os.path.abspath(gpu.__file__))).encode())
+    names = (C.c_char_p * 1)(b"lds_alloc_sequence")
+    mod, k = C.c_void_p(), C.c_void_p()
+    assert hip.gern_hip_compile(src, names, 1, opts, 1, None, C.byref(mod)) == 0, gpu._hip_error()
+    assert hip.gern_hip_get_kernel(mod, b"lds_alloc_sequence", C.byref(k)) == 0
+    out = torch.zeros(16, dtype=torch.int32, device="cuda")
+    lds = 8192
+    ptr, nbytes = C.c_void_p(out.data_ptr()), C.c_longlong(lds)
+    params = (C.c_void_p * 2)(C.cast(C.pointer(ptr), C.c_void_p), C.cast(C.pointer(nbytes), C.c_void_p))
+    grid, block = (C.c_uint32 * 3)(1, 1, 1), (C.c_uint32 * 3)(256, 1, 1)
+    assert hip.gern_hip_launch(k, grid, block, lds, params, None) == 0, gpu._hip_error()
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().tolist()
+    assert got[0:3] == [128, 128 + 1008, 128 + 1008 + 64]
+    assert got[3] == 1008 + 64 + 16
+    assert got[4] == 128 + 1008 + 64 + 16          # above c
+    assert got[5] == 128 + 1008                    # b's and c's space is back
+    assert got[6] == 128 and got[7] == 0           # everything released: the heap starts over
+    assert got[8] == 128 and got[9] == 1 and got[10] == 1
