@@ -452,34 +452,45 @@ def main():
         dC = torch.zeros((n, n), device="cuda")
         g = gern_amd.Gemm(variant, overwrite=True)  # config 4 is C = A * B
         t = measure(lambda: g(dA, dB, dC), 5, steps_gemm, torch, gern_amd)
+        vendor = {}
+        if variant == "bf16":
+            # The vendor library on the same operands, for comparison (not part of the product): torch.mm with fp32
+            # output is the same contract (bf16 in, fp32 accumulate, fp32 C); with bf16 output the library writes
+            # half the bytes.  This build's kernel and the library's are timed in turn, twice, each time with the
+            # same warm-up, and every kernel keeps its better turn: on a GPU whose clock follows its power draw
+            # and temperature, whichever runs second would otherwise pay for the first.
+            tA, tB = dA.view(torch.bfloat16), dB.view(torch.bfloat16)
+            out_bf16 = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+            calls = {"gemm_bf16_4096_vendor": lambda: torch.mm(tA, tB, out_dtype=torch.float32, out=dC),
+                     "gemm_bf16_4096_vendor_bf16_out": lambda: torch.mm(tA, tB, out=out_bf16)}
+            turns = {"ours": [t]}
+            for turn in range(2):
+                for name, call in calls.items():
+                    try:
+                        turns.setdefault(name, []).append(measure(call, 5, steps_gemm, torch, gern_amd))
+                    except Exception as e:  # a torch without out_dtype: say so, do not fail the benchmark
+                        vendor[name] = {"error": str(e)[:200]}
+                if turn == 0:
+                    turns["ours"].append(measure(lambda: g(dA, dB, dC), 5, steps_gemm, torch, gern_amd))
+            t = min(turns["ours"], key=lambda x: x["ms"])
+            for name in calls:
+                if name in turns:
+                    tv = min(turns[name], key=lambda x: x["ms"])
+                    tfv = 2.0 * n ** 3 / (tv["ms"] * 1e-3) / 1e12
+                    vendor[name] = {"TFLOP/s": tfv, "ms": tv["ms"], "ms_median": tv["ms_median"], "ms_min": tv["ms_min"],
+                                    "ms_turns": [x["ms"] for x in turns[name]],
+                                    "frac_peak": tfv / MFMA_BF16_PEAK_TFLOPS, "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS,
+                                    "what": "torch.mm (hipBLASLt), %s output; comparison only" % ("bf16" if name.endswith("bf16_out") else "fp32")}
         roof = roofline("gemm_%s_4096" % variant, table, bound, 2.0 * n ** 3, t, g)
         workloads["gemm_%s_4096" % variant] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
                                                "peak_TFLOP/s": roof["peak"], "roofline": roof}
         log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], roof["peak"]))
         if variant == "bf16":
-            # The vendor library on the same operands, same warm-up, same timing, for comparison (not part of the
-            # product): torch.mm with fp32 output is the same contract (bf16 in, fp32 accumulate, fp32 C);
-            # with bf16 output the library writes half the bytes.
-            tA, tB = dA.view(torch.bfloat16), dB.view(torch.bfloat16)
-            for name, out in (("gemm_bf16_4096_vendor", dC), ("gemm_bf16_4096_vendor_bf16_out", torch.empty((n, n), dtype=torch.bfloat16, device="cuda"))):
-                try:
-                    if out.dtype == torch.float32:
-                        call = lambda: torch.mm(tA, tB, out_dtype=torch.float32, out=out)  # noqa: E731
-                    else:
-                        call = lambda: torch.mm(tA, tB, out=out)  # noqa: E731
-                    tv = measure(call, 5, steps_gemm, torch, gern_amd)
-                except Exception as e:  # a torch without out_dtype: say so, do not fail the benchmark
-                    workloads[name] = {"error": str(e)[:200]}
-                    continue
-                tfv = 2.0 * n ** 3 / (tv["ms"] * 1e-3) / 1e12
-                workloads[name] = {"TFLOP/s": tfv, "ms": tv["ms"], "ms_median": tv["ms_median"], "ms_min": tv["ms_min"],
-                                   "frac_peak": tfv / MFMA_BF16_PEAK_TFLOPS, "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS,
-                                   "what": "torch.mm (hipBLASLt), %s output; comparison only" % ("fp32" if out.dtype == torch.float32 else "bf16")}
-                log("gemm bf16 4096^3, vendor library, %s out: %.1f us  %.1f TFLOP/s" % ("fp32" if out.dtype == torch.float32 else "bf16", tv["ms"] * 1e3, tfv))
-            # and once more this build's kernel, after the vendor's: the order of two measurements on a GPU whose clock follows its power draw
-            t2 = measure(lambda: g(dA, dB, dC), 5, steps_gemm, torch, gern_amd)
-            workloads["gemm_bf16_4096"]["ms_after_vendor"] = t2["ms"]
-            log("gemm bf16 4096^3 again: %.1f us" % (t2["ms"] * 1e3))
+            workloads["gemm_bf16_4096"]["ms_turns"] = [x["ms"] for x in turns["ours"]]
+            workloads.update(vendor)
+            for name, v in vendor.items():
+                if "ms" in v:
+                    log("%s: %.1f us  %.1f TFLOP/s (turns: %s)" % (name, v["ms"] * 1e3, v["TFLOP/s"], ", ".join("%.1f" % (x * 1e3) for x in v["ms_turns"])))
         if variant == "f32" and not args.no_cpu:
             from oracle import oracle as o
             from oracle import ref
@@ -531,9 +542,12 @@ def main():
         dA = torch.from_numpy(inputs.uniform((n, n), 4, -1.0, 1.0)).cuda()
         dB = torch.from_numpy(inputs.uniform((n, n), 5, -1.0, 1.0)).cuda()
         dC = torch.zeros((n, n), device="cuda")
-        for schedule, what in ((3, "block tiles staged through LDS one float per lane, 4x4 outputs per thread"),
-                               (6, "staged 16 bytes per lane"),
-                               (10, "block -> wavefront -> lane tiling, loads that write LDS directly, one output per lane")):
+        for schedule, what in ((3, "kernel_3.cu as the reference composes it: 64x64 block tiles staged through LDS one float per lane, "
+                                   "4x4 outputs per thread multiplied into C in global memory"),
+                               (6, "kernel_6.cu's composition plus a register stage of C: 64x64 block tiles, K tiles of 64 staged "
+                                   "16 bytes per lane, 4x4 outputs per thread in registers"),
+                               (10, "kernel_10.cu's block -> wavefront -> lane tiling with the lanes of a wavefront on consecutive "
+                                    "columns, loads that write LDS directly, one output per lane")):
             g = gern_amd.GemmSchedule(schedule)
             t = measure(lambda: g(dA, dB, dC), 3, MIN_SINGLE_LAUNCHES, torch, gern_amd)
             roof = roofline("gemm_schedule_kernel_%d_1024" % schedule, table, "fp32", 2.0 * n ** 3, t, g)

@@ -68,11 +68,13 @@ private:
 // reference's C += A * B) or written over it (C = A * B; C is never read).
 //   FMA    fp32 FMAs, 256 threads
 //   MFMA4  matrix cores, four wavefronts (any shape)
-//   MFMA8  matrix cores, eight wavefronts (the fast shape)
+//   MFMA8  matrix cores, eight wavefronts, 32 x 32 x 16 instruction
+//   MFMA16 matrix cores, eight wavefronts, 16 x 16 x 32 instruction (the fast shape; operands must be
+//          MatrixOperands that promise `exact`)
 //   MFMA8_F32  fp32 operands on the matrix cores, eight wavefronts
 class MatrixAccumulator : public AbstractDataType {
 public:
-    enum Engine { FMA, MFMA4, MFMA8, MFMA8_F32 };
+    enum Engine { FMA, MFMA4, MFMA8, MFMA8_F32, MFMA16 };
     MatrixAccumulator(const std::string &name, Engine engine, bool accumulate = true)
         : name(name), engine(engine), accumulate(accumulate) {
     }
@@ -101,6 +103,7 @@ public:
         return FunctionSignature{
             .name = engine == MFMA8_F32 ? "template load_acc_mfma8_f32" :
                     engine == MFMA8     ? "template load_acc_mfma8" :
+                    engine == MFMA16    ? "template load_acc_mfma16" :
                     engine == MFMA4     ? "template load_acc_mfma" :
                                           "template load_acc_fma",
             .args = {x, y},

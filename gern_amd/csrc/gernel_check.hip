@@ -67,6 +67,24 @@ __global__ void __launch_bounds__(512) check_gemm_bf16_8waves(gernels::MatrixBF1
 }
 template __global__ void check_gemm_bf16_8waves<256, 256, 4096>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32);
 
+template<int64_t BM, int64_t BN, int64_t KC, bool ADD>
+__global__ void __launch_bounds__(512) check_gemm_bf16_16x16x32(gernels::MatrixBF16 A, gernels::MatrixBF16 B, gernels::MatrixF32 C) {
+    const int64_t i = blockIdx.y * BM, j = blockIdx.x * BN;
+    auto acc = C.template load_acc_mfma16<BM, BN>(i, j);
+    for (int64_t k = 0; k < A.col; k += KC) {
+        auto a = A.template view_exact<BM, KC>(i, k);
+        auto b = B.template view_exact<KC, BN>(k, j);
+        gernels::matrix_multiply(a, b, acc);
+    }
+    if (ADD) {
+        C.add_acc(i, j, acc);
+    } else {
+        C.store_acc(i, j, acc);
+    }
+}
+template __global__ void check_gemm_bf16_16x16x32<256, 256, 4096, false>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32);
+template __global__ void check_gemm_bf16_16x16x32<256, 256, 4096, true>(gernels::MatrixBF16, gernels::MatrixBF16, gernels::MatrixF32);
+
 template<int64_t BM, int64_t BN, int64_t KC>
 __global__ void __launch_bounds__(256) check_gemm_f32(gernels::MatrixF32 A, gernels::MatrixF32 B, gernels::MatrixF32 C) {
     const int64_t i = blockIdx.y * BM, j = blockIdx.x * BN;

@@ -435,9 +435,15 @@ int gern_gemm_create(int variant, int flags, gern_pipeline *out) {
             // loads straight into LDS.  Those gernels keep their two stages in
             // static LDS (gernels/mm.h, mfma_direct / mfma_direct_f32): no dynamic LDS.
             gern_pipeline_s fast;
+            // bf16: the 16 x 16 x 32 matrix instruction (it draws less power than 32 x 32 x 16 for the same
+            // work, and the clock of this kernel is set by power); the other one stays selectable for
+            // comparison.
+            const bool wide_instruction = std::getenv("GERN_GEMM_BF16_32X32X16") != nullptr && experiments();
             rc = finish(&fast,
                         gemmProgram(element, true,
-                                    bf16 ? annot::MatrixAccumulator::MFMA8 : annot::MatrixAccumulator::MFMA8_F32,
+                                    !bf16            ? annot::MatrixAccumulator::MFMA8_F32 :
+                                    wide_instruction ? annot::MatrixAccumulator::MFMA8 :
+                                                       annot::MatrixAccumulator::MFMA16,
                                     accumulate, 256, 256, 512, 0),
                         flags);
             p->exact = std::move(fast.runner);

@@ -32,6 +32,7 @@ namespace gernels {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // Dynamic LDS of the kernel; the launch sizes it (Global(..., smem_size)).
@@ -114,7 +115,36 @@ struct MfmaAcc {
     static constexpr int TM = (int)(WM / 32);
     static constexpr int TN = (int)(WN / 32);
     static constexpr int threads = NW * kWaveSize;
+    static constexpr int kTile = 32;            // edge of the matrix instruction's result
     f32x16_t acc[TM][TN];
+
+    __device__ __forceinline__ void destroy() {
+    }
+};
+
+// The accumulators of the fast bf16 path: a 256 x 256 tile on eight wavefronts
+// (2 x 4, 128 rows x 64 columns each) as 8 x 4 results of
+// v_mfma_f32_16x16x32_bf16, computed TRANSPOSED (B's fragment is the
+// instruction's first operand): acc[tm][tn][i] of lane l is row
+// 128 wm + 16 tm + l % 16, column 64 wn + 16 tn + 4 (l / 16) + i, four
+// consecutive columns of C per lane and tile (16-byte stores).
+//
+// The 16 x 16 x 32 instruction does the work of the 32 x 32 x 16 one in the
+// same number of cycles (a loop of nothing but matrix instructions on random
+// operands runs both at 1024 flop per cycle and SIMD) but DRAWS LESS POWER, and
+// power is what sets the clock of a kernel like this one: that loop settles at
+// 2.05-2.1 GHz with 16 x 16 x 32 and at 1.78-1.85 GHz with 32 x 32 x 16.
+template<int64_t BM, int64_t BN>
+struct MfmaAcc16 {
+    static_assert(BM == 256 && BN == 256, "written for 256 x 256 tiles");
+    static constexpr int WC = 4;
+    static constexpr int64_t WM = 128;
+    static constexpr int64_t WN = 64;
+    static constexpr int TM = 8;
+    static constexpr int TN = 4;
+    static constexpr int threads = 8 * kWaveSize;
+    static constexpr int kTile = 16;
+    f32x4_t acc[TM][TN];
 
     __device__ __forceinline__ void destroy() {
     }
@@ -200,6 +230,82 @@ __device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const
     detail::write_acc<false>(*this, x, y, t);
 }
 
+namespace detail {
+
+// ADD: C += tile (read-modify-write); otherwise C = tile.
+template<bool ADD, int64_t BM, int64_t BN>
+__device__ __forceinline__ void write_acc16(const MatrixF32 &m, int64_t x, int64_t y, const MfmaAcc16<BM, BN> &t) {
+    using Acc = MfmaAcc16<BM, BN>;
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int64_t r0 = x + (int64_t)(w / Acc::WC) * Acc::WM + (lane % 16);
+    const int64_t c0 = y + (int64_t)(w % Acc::WC) * Acc::WN + 4 * (lane / 16);
+    // workgroup-uniform: every group of four columns starts on a 16-byte boundary
+    const bool aligned = ((((uint64_t)m.data) & 15u) == 0) && (m.lda % 4 == 0) && (y % 4 == 0);
+    const int64_t span = (m.row - 1) * m.lda + m.col;
+#pragma unroll
+    for (int tm = 0; tm < Acc::TM; tm++) {
+        const int64_t rr = r0 + tm * 16;
+        if (rr >= m.row) {
+            continue;
+        }
+        // the two tiles of a pair of tn fill the same 128-byte lines: back to back
+#pragma unroll
+        for (int tn = 0; tn < Acc::TN; tn++) {
+            const int64_t cc = c0 + tn * 16;
+            const f32x4_t a = t.acc[tm][tn];
+            float *p = m.data + rr * m.lda + cc;
+            if (aligned && cc + 3 < m.col) {
+                float4 v = make_float4(a[0], a[1], a[2], a[3]);
+                if (ADD) {
+                    const float4 o = *reinterpret_cast<const float4 *>(p);
+                    v = make_float4(o.x + v.x, o.y + v.y, o.z + v.z, o.w + v.w);
+                    *reinterpret_cast<float4 *>(p) = v;
+                } else {
+                    // written once, never re-read by this kernel
+                    store_result16<kThroughStores>(m.data, span, rr * m.lda + cc, v);
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (cc + q < m.col) {
+                        if (ADD) {
+                            p[q] += a[q];
+                        } else {
+                            store_result4<kThroughStores>(m.data, span, rr * m.lda + cc + q, a[q]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace detail
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ MfmaAcc16<BM, BN> MatrixF32::load_acc_mfma16(int64_t, int64_t) const {
+    MfmaAcc16<BM, BN> t;
+#pragma unroll
+    for (int tm = 0; tm < MfmaAcc16<BM, BN>::TM; tm++) {
+#pragma unroll
+        for (int tn = 0; tn < MfmaAcc16<BM, BN>::TN; tn++) {
+            t.acc[tm][tn] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    return t;
+}
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::add_acc(int64_t x, int64_t y, const MfmaAcc16<BM, BN> &t) const {
+    detail::write_acc16<true>(*this, x, y, t);
+}
+
+template<int64_t BM, int64_t BN>
+__device__ __forceinline__ void MatrixF32::store_acc(int64_t x, int64_t y, const MfmaAcc16<BM, BN> &t) const {
+    detail::write_acc16<false>(*this, x, y, t);
+}
+
 constexpr int kMfmaBK = 64;                      // K depth of one LDS stage
 constexpr int64_t kMfmaMaxLd = 1 << 20;          // direct-to-LDS paths: largest row pitch of A and B, in elements
 constexpr int kMfmaRowBytes = 2 * kMfmaBK + 16;  // padded LDS row: 144 bytes
@@ -240,13 +346,13 @@ namespace detail {
 // stage 167; two wavefront groups half a stage out of phase (one computing
 // while the other moves data) 140; this one, with 64-bit lane addresses, 131;
 // as it is, 116-124.
-template<int64_t BM, int64_t BN, int64_t KC>
+template<int64_t BM, int64_t BN, int64_t KC, typename Acc>
 __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, true> &A,
-                                            const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc<BM, BN, 8> &C) {
-    using Acc = MfmaAcc<BM, BN, 8>;
-    static_assert(BM == 256 && BN == 256, "written for 256 x 256 tiles");
+                                            const GlobalView<KC, BN, uint16_t, true> &B, Acc &C) {
+    static_assert(BM == 256 && BN == 256 && Acc::threads == 512 && Acc::WC == 4, "written for 256 x 256 tiles on eight wavefronts");
     constexpr int TM = Acc::TM, TN = Acc::TN;
-    constexpr int KSTEPS = kMfmaBK / 16;
+    constexpr bool k16 = Acc::kTile == 16;  // v_mfma_f32_16x16x32_bf16 (MfmaAcc16) or v_mfma_f32_32x32x16_bf16 (MfmaAcc)
+    constexpr int KSTEPS = kMfmaBK / (k16 ? 32 : 16);
     constexpr int A_BYTES = 256 * 128;
     constexpr int STAGE = A_BYTES + 64 * 512;
     typedef short v4s_t __attribute__((ext_vector_type(4)));
@@ -295,7 +401,10 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     for (int odd = 0; odd < 2; odd++) {
         // B slot: K row 2 i + lane / 32, position lane % 32, holds chunk
         // (lane % 32) ^ (4 * (K row & 3)); the K row's parity class is that of j
-        const int chunk_b = (lane % 32) ^ (4 * ((2 * odd + lane / 32) & 3));
+        // (16 x 16 x 32: also ^ 2 where bit 3 of the K row is set, which is the parity of the wavefront:
+        // the K row is 8 w + 2 j + lane / 32.  The two groups of sixteen lanes that one pass of a
+        // transposing read serves then address K rows 8 apart, and would meet in the same banks.)
+        const int chunk_b = (lane % 32) ^ (4 * ((2 * odd + lane / 32) & 3)) ^ (k16 ? 2 * (wu & 1) : 0);
         lane_off_b[odd] = ((lane / 32) * (int)B.lda + (chunk_b < last_chunk_b ? chunk_b : last_chunk_b) * 8) * 2;
     }
     // Raw 32-bit buffer descriptors whose num_records end at the last valid
@@ -344,29 +453,33 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         }
     };
 
-    // A fragment of this lane: row lane % 32 of each 32-row tile, K block
+    // 32 x 32 x 16.  A fragment of this lane: row lane % 32 of each 32-row tile, K block
     // 2 s + lane / 32 of K step s.
-    const int a_row_off = ((w / Acc::WC) * (int)Acc::WM + (lane % 32)) * 128;
-    const int a_swz = ((lane % 32) >> 1) & 7;
-    const int a_half = lane / 32;
-    // B fragment: lane p of 16-lane group g addresses K row 16 s + 8 (g / 2) +
+    // 16 x 16 x 32.  Row lane % 16 of each 16-row tile, K block 4 s + lane / 16 of K step s (32 deep).
+    constexpr int kRows = k16 ? 16 : 32;  // rows of A (columns of B) per instruction
+    const int a_row_off = ((w / Acc::WC) * (int)Acc::WM + (lane % kRows)) * 128;
+    const int a_swz = ((lane % kRows) >> 1) & 7;
+    const int a_part = lane / kRows;
+    // B fragment, 32 x 32 x 16: lane p of 16-lane group g addresses K row 16 s + 8 (g / 2) +
     // 4 q + p / 4, columns 16 (g % 2) + 4 (p % 4) .. + 3 of the 32-column tile;
     // the transposing read hands it K rows 8 (g / 2) + 4 q .. + 3 of column
     // 16 (g % 2) + p, which is what MFMA lane 16 g + p holds.
+    // 16 x 16 x 32: K row 32 s + 8 g + 4 q + p / 4, columns 4 (p % 4) .. + 3 of the 16-column tile; the
+    // read hands it K rows 8 g + 4 q .. + 3 of column p.
     const int g = lane / 16, p = lane % 16;
-    const int b_col0 = (w % Acc::WC) * (int)Acc::WN + 16 * (g % 2);
-    const int b_krow = 8 * (g / 2) + p / 4;
-    const int b_swz = 4 * (p / 4);  // (k & 3) == p / 4: the other terms are multiples of 4
+    const int b_col0 = (w % Acc::WC) * (int)Acc::WN + (k16 ? 0 : 16 * (g % 2));
+    const int b_krow = (k16 ? 8 * g : 8 * (g / 2)) + p / 4;
+    const int b_swz = (4 * (p / 4)) ^ (k16 ? 2 * (g & 1) : 0);  // (k & 3) == p / 4: the other terms are multiples of 4
     // Every LDS address below is ONE offset from the stage array: the compiler
     // tells the two stages apart only through short pointer chains.
     auto load_a = [&](const unsigned char *stage, int tm, int s) {
-        const int pos = (2 * s + a_half) ^ a_swz;
-        const int at = a_row_off + tm * 32 * 128 + pos * 16;
+        const int pos = ((k16 ? 4 : 2) * s + a_part) ^ a_swz;
+        const int at = a_row_off + tm * kRows * 128 + pos * 16;
         return *reinterpret_cast<const bf16x8_t *>(stage + at);
     };
     auto load_b = [&](const unsigned char *stage, int tn, int s) {
-        const int chunk = ((b_col0 + tn * 32) / 8 + (p % 4) / 2) ^ b_swz;
-        const int at = A_BYTES + (16 * s + b_krow) * 512 + chunk * 16 + (p % 2) * 8;
+        const int chunk = ((b_col0 + tn * kRows) / 8 + (p % 4) / 2) ^ b_swz;
+        const int at = A_BYTES + ((k16 ? 32 : 16) * s + b_krow) * 512 + chunk * 16 + (p % 2) * 8;
         const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + at));
         const v4s_t hi =
             __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + (at + 4 * 512)));
@@ -374,33 +487,74 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         return __builtin_bit_cast(bf16x8_t, both);
     };
     auto compute = [&](const unsigned char *stage) {
-        bf16x8_t af[2][TM], bfr[2][TN];
+        if constexpr (k16) {
+            // Four phases per stage: (K step, upper or lower four row tiles).  The fragments of the next
+            // phase are read while the sixteen instructions of this one run.
+            constexpr int HALF = TM / 2;
+            bf16x8_t af[2][HALF], bfr[2][TN];
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++) {
-            af[0][tm] = load_a(stage, tm, 0);
-        }
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++) {
-            bfr[0][tn] = load_b(stage, tn, 0);
-        }
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            const int cur = s & 1, nxt = cur ^ 1;
-            if (s + 1 < KSTEPS) {
-#pragma unroll
-                for (int tm = 0; tm < TM; tm++) {
-                    af[nxt][tm] = load_a(stage, tm, s + 1);
-                }
-#pragma unroll
-                for (int tn = 0; tn < TN; tn++) {
-                    bfr[nxt][tn] = load_b(stage, tn, s + 1);
-                }
+            for (int t = 0; t < HALF; t++) {
+                af[0][t] = load_a(stage, t, 0);
             }
 #pragma unroll
-            for (int tm = 0; tm < TM; tm++) {
+            for (int tn = 0; tn < TN; tn++) {
+                bfr[0][tn] = load_b(stage, tn, 0);
+            }
 #pragma unroll
-                for (int tn = 0; tn < TN; tn++) {
-                    C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][tm], bfr[cur][tn], C.acc[tm][tn], 0, 0, 0);
+            for (int ph = 0; ph < 2 * KSTEPS; ph++) {
+                const int s = ph / 2, h = ph % 2;
+                if (ph + 1 < 2 * KSTEPS) {
+                    const int ns = (ph + 1) / 2, nh = (ph + 1) % 2;
+#pragma unroll
+                    for (int t = 0; t < HALF; t++) {
+                        af[(ph + 1) & 1][t] = load_a(stage, nh * HALF + t, ns);
+                    }
+                    if (nh == 0) {
+#pragma unroll
+                        for (int tn = 0; tn < TN; tn++) {
+                            bfr[ns & 1][tn] = load_b(stage, tn, ns);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < HALF; t++) {
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        // transposed: B's fragment first, so that a lane ends up with four consecutive columns
+                        C.acc[h * HALF + t][tn] =
+                            __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[s & 1][tn], af[ph & 1][t], C.acc[h * HALF + t][tn], 0, 0, 0);
+                    }
+                }
+            }
+        } else {
+            bf16x8_t af[2][TM], bfr[2][TN];
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++) {
+                af[0][tm] = load_a(stage, tm, 0);
+            }
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++) {
+                bfr[0][tn] = load_b(stage, tn, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++) {
+                const int cur = s & 1, nxt = cur ^ 1;
+                if (s + 1 < KSTEPS) {
+#pragma unroll
+                    for (int tm = 0; tm < TM; tm++) {
+                        af[nxt][tm] = load_a(stage, tm, s + 1);
+                    }
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        bfr[nxt][tn] = load_b(stage, tn, s + 1);
+                    }
+                }
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++) {
+#pragma unroll
+                    for (int tn = 0; tn < TN; tn++) {
+                        C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[cur][tm], bfr[cur][tn], C.acc[tm][tn], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -431,6 +585,12 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
 }
 
 }  // namespace detail
+
+template<int64_t BM, int64_t BN, int64_t KC>
+__device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t, true> &A,
+                                                const GlobalView<KC, BN, uint16_t, true> &B, MfmaAcc16<BM, BN> &C) {
+    detail::mfma_direct(A, B, C);
+}
 
 template<int64_t BM, int64_t BN, int64_t KC, int NW, bool EXACT>
 __device__ __forceinline__ void matrix_multiply(const GlobalView<BM, KC, uint16_t, EXACT> &A,

@@ -107,6 +107,8 @@ struct GlobalView;
 template<int64_t BM, int64_t BN, int NW>
 struct MfmaAcc;
 template<int64_t BM, int64_t BN>
+struct MfmaAcc16;
+template<int64_t BM, int64_t BN>
 struct FmaAcc;
 template<int64_t BM, int64_t BN>
 struct MfmaAccF32;
@@ -149,6 +151,12 @@ struct MatrixF32 {
     __device__ __forceinline__ void add_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const;
     template<int64_t BM, int64_t BN, int NW>
     __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAcc<BM, BN, NW> &t) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ MfmaAcc16<BM, BN> load_acc_mfma16(int64_t x, int64_t y) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void add_acc(int64_t x, int64_t y, const MfmaAcc16<BM, BN> &t) const;
+    template<int64_t BM, int64_t BN>
+    __device__ __forceinline__ void store_acc(int64_t x, int64_t y, const MfmaAcc16<BM, BN> &t) const;
     template<int64_t BM, int64_t BN>
     __device__ __forceinline__ FmaAcc<BM, BN> load_acc_fma(int64_t x, int64_t y) const;
     template<int64_t BM, int64_t BN>
