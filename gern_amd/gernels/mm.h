@@ -318,9 +318,10 @@ constexpr int64_t mfma_lds_bytes() {
 
 namespace detail {
 
-// The fast bf16 path: 256 x 256 tile, eight wavefronts; K a multiple of the
-// 64-deep stage, the column count of B a multiple of 8; tiles at the bottom
-// and right edges of C may be partial.
+// The fast bf16 path: 256 x 256 tile, eight wavefronts, for either accumulator
+// type (MfmaAcc16: v_mfma_f32_16x16x32_bf16, the one the pipeline uses;
+// MfmaAcc<.., 8>: v_mfma_f32_32x32x16_bf16); tiles at the bottom and right
+// edges of C may be partial, and so may the last stage of K.
 //
 // Both operands go from global memory STRAIGHT INTO LDS (buffer_load ... lds, 16
 // bytes per lane, no register round trip, no LDS write instructions), two
@@ -345,7 +346,19 @@ namespace detail {
 // Measured alternatives at 4096^3 (us): register-staged with one barrier per
 // stage 167; two wavefront groups half a stage out of phase (one computing
 // while the other moves data) 140; this one, with 64-bit lane addresses, 131;
-// as it is, 116-124.
+// on v_mfma_f32_32x32x16_bf16 (MfmaAcc) 116-120; on v_mfma_f32_16x16x32_bf16
+// (MfmaAcc16) 104-109.
+//
+// THE KERNEL IS BOUND BY POWER, not by issue slots: the two instructions need
+// the same number of cycles (246 500 and 250 800 per launch and XCD, counted by
+// GRBM_GUI_ACTIVE), but the clock settles at 2.05 GHz with the first and at
+// 2.28 GHz with the second, and the time follows the clock.  Variants that
+// change the schedule and not the work leave the time where it is: the K loop
+// rotated so that the barrier stands before a stage's last sixteen
+// instructions (they cover the wait for the next stage's first fragments)
+// takes 4 % MORE cycles at a 3 % higher clock; C stored in whole 128-byte
+// lines (lanes p and p ^ 8 swapping a piece through DPP) instead of 64-byte
+// halves: no difference.
 template<int64_t BM, int64_t BN, int64_t KC, typename Acc>
 __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, true> &A,
                                             const GlobalView<KC, BN, uint16_t, true> &B, Acc &C) {

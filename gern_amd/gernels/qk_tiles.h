@@ -30,11 +30,11 @@
 // thus spread over just two lanes (l and l + 32): its maximum and its sum are
 // 128 operations inside a lane and ONE exchange between the two, no DPP
 // butterflies, and the four scores b = 0 .. 3 are consecutive columns of S, one
-// 16-byte store.  (The 16 x 16 x 32 instruction, whose accumulators put a row
-// on sixteen lanes with four columns each, runs at HALF the rate on this GPU --
-// measured with loops of nothing but MFMAs: 1.23 against 2.46 PFLOP/s at
-// 2.4 GHz -- and the butterflies over sixteen lanes were a third of the
-// vector-ALU work of the softmax.)
+// 16-byte store.  (With the 16 x 16 x 32 instruction, whose accumulators put a
+// row on sixteen lanes with four columns each, the butterflies over sixteen
+// lanes were a third of the vector-ALU work of the softmax.  The two
+// instructions do the same work per cycle; the products of this kernel wait
+// for their operands, not for the matrix pipe, with either.)
 //
 // The exchange.  An entry is one 64-bit word per (row, column block): s in the
 // upper half, below it m as a sixteen-bit integer (a row is shifted by
