@@ -281,8 +281,8 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
         return fail("gern_softmax_create: null argument");
     }
     *out = nullptr;
-    if (ncol < 1 || ncol > 8192 || rows_per_wave < 1) {
-        return fail("gern_softmax_create: ncol must be in [1, 8192] and rows_per_wave positive");
+    if (ncol < 1 || ncol > GERN_SOFTMAX_MAX_COLS || rows_per_wave < 1) {
+        return fail("gern_softmax_create: ncol must be in [1, GERN_SOFTMAX_MAX_COLS = 65536] and rows_per_wave positive");
     }
     // A row is cut into equal pieces of whole 256-column chunks, at least 512
     // columns each, one per wavefront of the workgroup that owns the row (8, 4
@@ -290,6 +290,9 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
     // the stores of another (8192 x 4096: 46 -> 39.5 us, 4096 x 8192: 68 -> 41.5;
     // sixteen wavefronts of 256 columns: 54 us).  Widths that do not divide
     // that way keep one wavefront per row.
+    // A row wider than 8192 columns does not fit the registers of one wavefront (32 chunks of 256 columns,
+    // 128 values per lane): it is cut into 4, 8 or 16 pieces of at most 4096 columns, whatever its width (the
+    // last pieces of a width that does not divide are partly or wholly unused, gernels/softmax.h BlockTile).
     int64_t waves = 1;
     for (int64_t w : {8, 4, 2}) {
         if (ncol % (w * 256) == 0 && ncol / w >= 512) {
@@ -297,13 +300,16 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
             break;
         }
     }
+    if (ncol > 8192) {
+        waves = ncol <= 16384 ? 4 : ncol <= 32768 ? 8 : 16;
+    }
     if (const char *forced = std::getenv("GERN_SOFTMAX_WAVES"); forced != nullptr && experiments()) {
         waves = std::atoll(forced);
         if ((waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) || ncol % (4 * waves) != 0) {
             return fail("GERN_SOFTMAX_WAVES must be 1, 2, 4, 8 or 16 and divide the row into 16-byte pieces");
         }
     }
-    if (rows_per_wave * ((ncol / waves + 255) / 256) > 32) {
+    if (rows_per_wave * (((ncol + waves - 1) / waves + 255) / 256) > 32) {
         return fail("gern_softmax_create: a wavefront holds at most 32 x 256 columns of rows in registers");
     }
     auto p = std::make_unique<gern_pipeline_s>();
@@ -549,14 +555,19 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
     if (head_dim < 32 || head_dim > 256 || head_dim % 32 != 0) {
         return fail("gern_qk_softmax_create: head_dim must be a multiple of 32 in [32, 256]");
     }
-    if (max_keys < 256 || max_keys > 4096 || max_keys % 256 != 0) {
-        return fail("gern_qk_softmax_create: max_keys must be a multiple of 256 in [256, 4096]");
+    // The tile kernel holds one 256-column piece of a row per workgroup, whatever the row's width; the
+    // row-block kernel keeps sixteen whole rows in the registers of one workgroup.
+    const bool tiles = head_dim % 64 == 0 && !(flags & GERN_PIPELINE_QK_ROW_BLOCKS);
+    if (max_keys < 256 || max_keys > (tiles ? GERN_QK_MAX_KEYS : 4096) || max_keys % 256 != 0) {
+        return fail(tiles ? "gern_qk_softmax_create: max_keys must be a multiple of 256 in [256, GERN_QK_MAX_KEYS = 65536]"
+                          : "gern_qk_softmax_create: max_keys must be a multiple of 256 in [256, 4096] for head dimensions that are not "
+                            "multiples of 64 (and with GERN_PIPELINE_QK_ROW_BLOCKS)");
     }
     auto p = std::make_unique<gern_pipeline_s>();
     p->kind = gern_pipeline_s::QK_SOFTMAX;
     p->head_dim = head_dim;
     p->ncol = max_keys;
-    p->qk_tiles = head_dim % 64 == 0 && !(flags & GERN_PIPELINE_QK_ROW_BLOCKS);
+    p->qk_tiles = tiles;
     try {
         auto Q = AbstractDataTypePtr(new const annot::MatrixOperand("Q", annot::MatrixOperand::BF16));
         auto K = AbstractDataTypePtr(new const annot::MatrixOperand("K", annot::MatrixOperand::BF16));
@@ -683,7 +694,8 @@ __attribute__((visibility("hidden"))) int gern_detail_qk_softmax_run(gern_pipeli
         const int64_t pitch = ((N + 255) / 256 + 15) / 16 * 16;
         const int64_t capacity = ((int64_t)GERN_QK_SCRATCH_BYTES - 256) / 8;
         if (scratch == nullptr || padded_rows * pitch > capacity) {
-            return fail(name + ": M x N needs more than GERN_QK_SCRATCH_BYTES of exchange memory (M up to 16384 at 4096 keys)");
+            return fail(name + ": M x N needs more than GERN_QK_SCRATCH_BYTES of exchange memory (M up to 16384 at 4096 keys, "
+                               "8192 at 8192, 1024 at 65536)");
         }
         int32_t spin_limit = 0;
         if (!qkSpinLimit(&spin_limit)) {

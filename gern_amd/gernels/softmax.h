@@ -158,14 +158,27 @@ __device__ __forceinline__ void divide_vec(const TV &vec, const T &in, T &out) {
 // that start and end at different times, so loads and stores of different
 // rows overlap; one wavefront per 4096-column row keeps 64 values per lane,
 // leaves room for three wavefronts per SIMD, and measures 20 % slower.
+//
+// A width that does not divide into NW whole 16-byte pieces is cut into pieces
+// of wave_cols = ceil(C / NW) rounded up to whole 256-column chunks; the last
+// wavefronts then use only part of their piece, or none of it.
 template<int64_t R, int64_t C, int NW>
 struct BlockTile {
-    static_assert(NW >= 1 && C % (4 * NW) == 0, "whole 16-byte pieces per wavefront");
+    static_assert(NW >= 1 && C >= 1, "at least one wavefront and one column");
     static constexpr int64_t rows = R;
     static constexpr int64_t cols = C;
     static constexpr int waves = NW;
-    static constexpr int64_t wave_cols = C / NW;
-    WaveTile<R, C / NW> part;
+    static constexpr int64_t wave_cols = C % (4 * NW) == 0 ? C / NW : ((C + NW - 1) / NW + kWaveCols - 1) / kWaveCols * kWaveCols;
+    static constexpr bool even = wave_cols * NW == C;
+    WaveTile<R, wave_cols> part;
+
+    // Wavefronts 0 .. full - 1 use their whole piece, wavefront `full` the first `rest` columns of its piece
+    // (if any), the wavefronts after it nothing.
+    static constexpr int full = (int)(C / wave_cols);
+    static constexpr int64_t rest = C - full * wave_cols;
+    static __device__ __forceinline__ int64_t used_by(int w) {
+        return even || w < full ? wave_cols : (w == full ? rest : 0);
+    }
 
     __device__ __forceinline__ void destroy() {
     }
@@ -184,9 +197,32 @@ GERN_BLOCK_ALLOCATOR(16)
 
 template<int NW, int64_t R, int64_t C>
 __device__ __forceinline__ BlockTile<R, C, NW> MatrixF32::load_block(int64_t x, int64_t y) const {
-    BlockTile<R, C, NW> t;
-    const int w = (int)(threadIdx.x / kWaveSize);
-    t.part = load_wave<R, C / NW>(x, y + w * (C / NW));
+    using T = BlockTile<R, C, NW>;
+    T t;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
+    t.part = load_wave<R, T::wave_cols>(x, y + w * T::wave_cols);
+    if constexpr (!T::even) {
+        // The columns of a piece that are not in use (whatever the matrix holds there) become -infinity: no
+        // row maximum takes it, and its exponential adds nothing to a row sum, so that every later stage runs
+        // the same code on every wavefront; only the store needs the width again.  One code path on purpose:
+        // separate instances per wavefront for the reductions keep a second copy of the tile alive where the
+        // paths meet (16 chunks per lane: 282 registers spilled).
+        const int left0 = (int)T::used_by(w) - 4 * lane_id();
+        const float none = -__builtin_huge_valf();
+#pragma unroll
+        for (int64_t r = 0; r < R; r++) {
+#pragma unroll
+            for (int64_t k = 0; k < WaveTile<R, T::wave_cols>::chunks; k++) {
+                const int left = left0 - (int)(k * kWaveCols);
+                float4 v = t.part.v[r][k];
+                v.x = 0 < left ? v.x : none;
+                v.y = 1 < left ? v.y : none;
+                v.z = 2 < left ? v.z : none;
+                v.w = 3 < left ? v.w : none;
+                t.part.v[r][k] = v;
+            }
+        }
+    }
     return t;
 }
 
@@ -197,8 +233,18 @@ __device__ __forceinline__ BlockTile<R, C, NW> MatrixF32::view_block(int64_t, in
 
 template<int64_t R, int64_t C, int NW>
 __device__ __forceinline__ void MatrixF32::store_block(int64_t x, int64_t y, const BlockTile<R, C, NW> &t) const {
-    const int w = (int)(threadIdx.x / kWaveSize);
-    store_wave(x, y + w * (C / NW), t.part);
+    using T = BlockTile<R, C, NW>;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
+    if constexpr (T::even) {
+        store_wave(x, y + w * T::wave_cols, t.part);
+    } else {
+        // The tile ends at column y + C: stored through a copy of the matrix that ends there too, so that the
+        // one bounds test every store has anyway does the clipping (a width passed to store_wave as a run-time
+        // value costs the kernel 85 registers).
+        MatrixF32 clipped = *this;
+        clipped.col = y + C < col ? y + C : col;
+        clipped.store_wave(x, y + w * T::wave_cols, t.part);
+    }
 }
 
 namespace detail {
@@ -210,8 +256,9 @@ namespace detail {
 // wavefront may start the second while another still reads the first.
 template<typename Op, typename TV, int64_t R, int64_t C, int NW>
 __device__ __forceinline__ void reduce_block_rows(TV &out, const BlockTile<R, C, NW> &in, float *scratch) {
+    // (columns of a piece that are not in use hold -infinity, then 0 after the exponential: see load_block)
     reduce_rows<Op>(out, in.part);
-    const int w = (int)(threadIdx.x / kWaveSize);
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWaveSize));
     if (lane_id() == 0) {
 #pragma unroll
         for (int64_t r = 0; r < R; r++) {

@@ -83,11 +83,15 @@ int gern_blur_chain_run(gern_pipeline p, const float *in, int64_t rows, int64_t 
                         float *out, int64_t ld_out, void *stream);
 
 /* Row-wise numerically stable softmax over matrices with exactly `ncol`
- * columns: max, x - max, exp, sum, divide, fused; a workgroup holds
- * rows_per_wave rows in registers, in one wavefront or, for rows of 1024
- * columns and more that divide into 256-column chunks, spread over 2, 4 or 8
- * wavefronts.  The five calls are the reference's softmax gernels,
- * apps/common/annot/functions.h:9-173. */
+ * columns (1 .. GERN_SOFTMAX_MAX_COLS): max, x - max, exp, sum, divide, fused;
+ * a workgroup holds rows_per_wave rows in registers, in one wavefront or, for
+ * rows of 1024 columns and more that divide into 256-column chunks, spread
+ * over 2, 4 or 8 wavefronts; rows wider than 8192 columns, of any width, are
+ * spread over 4, 8 or 16 wavefronts (rows_per_wave must then be 1).  The
+ * reference's row reductions likewise share a row among `stride` threads and
+ * meet in shared memory (apps/common/impl/impl.h:80-188).  The five calls are
+ * the reference's softmax gernels, apps/common/annot/functions.h:9-173. */
+#define GERN_SOFTMAX_MAX_COLS 65536
 int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pipeline *out);
 int gern_softmax_run(gern_pipeline p, const float *in, float *out, int64_t rows, int64_t ld,
                      void *stream);
@@ -115,12 +119,14 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
  * patterns), S is M x N fp32; MFMA tiles feed an in-register row reduction.
  * Q and K 16-byte aligned.
  * head_dim = D (a multiple of 32, at most 256); max_keys bounds N (a multiple
- * of 256, at most 4096).
+ * of 256, at most GERN_QK_MAX_KEYS when D is a multiple of 64, else 4096).
  * D a multiple of 64: one workgroup per 256 x 256 tile of S; the workgroups
  * of a row block exchange their row maxima and sums through
  * GERN_QK_SCRATCH_BYTES of device memory that create allocates (the only device
  * memory this library allocates) and the tiles wait in registers meanwhile.
- * M x N must fit that memory; runs of ONE pipeline must not overlap in time
+ * M x N must fit that memory (8 bytes per row and 256 keys, keys rounded up
+ * to a multiple of 4096: M up to 16384 at 4096 keys, 8192 at 8192 keys, 1024
+ * at 65536); runs of ONE pipeline must not overlap in time
  * (launch them on one stream, or order the streams).  A wavefront that waits
  * in vain for the rest of its row block (after a second or so: the launch
  * shares the GPU with something that keeps its partners from starting) stores
@@ -133,6 +139,7 @@ int gern_gemm_run(gern_pipeline p, const void *A, const void *B, float *C, int64
  * workgroup, logits in accumulators, no device memory besides Q, K and S.
  * No counterpart in the reference (it has no bf16 and no matrix-core path);
  * the softmax stages are those of apps/common/annot/functions.h:9-173. */
+#define GERN_QK_MAX_KEYS 65536
 int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_pipeline *out);
 int gern_qk_softmax_run(gern_pipeline p, const uint16_t *Q, const uint16_t *K, float *S, int64_t M,
                         int64_t N, float scale, void *stream);

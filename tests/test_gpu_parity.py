@@ -190,6 +190,57 @@ def test_softmax_matches_oracle(gpu, oracle, shape, kw):
     assert np.max(np.abs(got - want) / want) < 1e-5
 
 
+# Rows wider than 8192 columns are cut into 4, 8 or 16 pieces of at most 4096 columns, one per wavefront;
+# widths that do not divide leave the last pieces partly used (8200 -> 4 x 2052, the last 2044; 20000 -> 8 x
+# 2500; 40004 -> 16 x 2504, the last 2444; 8193 -> 4 x 2052, the last 2037).  The oracle adds a row left to right in fp32, as the reference's CPU
+# code does, and over this many terms strays from the exact sum by more than the bar itself: the result is held
+# to 1e-5 against the exact (fp64) softmax, and to the oracle within 1e-5 plus the oracle's own distance from it.
+@pytest.mark.parametrize("shape", [(5, 8193), (9, 8200), (6, 12288), (33, 16384), (3, 20000), (4, 32768), (2, 40004),
+                                   (3, 65536), (1, 65531)])
+def test_softmax_rows_wider_than_one_wavefront_holds(gpu, oracle, shape):
+    x = oracle.normal(shape, 23 + shape[1] % 97, 0.0, 2.0)
+    got = _run_softmax(gpu, x)
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    exact = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(got - exact) / exact) < 1e-5, shape
+    want = oracle.softmax_rows(x)
+    own = float(np.max(np.abs(want - exact) / exact))
+    assert np.max(np.abs(got - want) / want) < 1e-5 + own, (shape, own)
+    assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
+    assert np.all(got.argmax(axis=1) == x.argmax(axis=1))
+
+
+def test_softmax_wide_rows_in_a_window_and_with_a_wide_range(gpu, oracle):
+    import torch
+    # a 9000-column window of a wider buffer: the unused part of the last piece lies INSIDE the buffer
+    ncol, ld, c0 = 9000, 9300, 4
+    x = oracle.normal((7, ld), 29, 0.0, 2.0)
+    x[:, c0 + ncol:] = 50.0  # would win every maximum if a reduction read past the window
+    dx = _dev(x)
+    dy = torch.full((7, ld), -7.0, dtype=torch.float32, device="cuda")
+    gpu.Softmax(ncol)(dx[:, c0:c0 + ncol], dy[:, c0:c0 + ncol])
+    torch.cuda.synchronize()
+    got = dy.cpu().numpy()
+    x64 = x[:, c0:c0 + ncol].astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    exact = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(got[:, c0:c0 + ncol] - exact) / exact) < 1e-5
+    got[:, c0:c0 + ncol] = -7.0
+    assert np.all(got == -7.0)
+    # differences of more than 87 from the row maximum on a wide row
+    x = oracle.normal((3, 10000), 31, 0.0, 40.0)
+    got = _run_softmax(gpu, x)
+    want = oracle.softmax_rows(x)
+    big = want >= 1e-30
+    assert np.max(np.abs(got[big] - want[big]) / want[big]) < 1e-5
+    assert np.max(np.abs(got[~big] - want[~big])) < 1e-35
+    with pytest.raises(gpu.GernError, match="65536"):
+        gpu.Softmax(65537)
+    with pytest.raises(gpu.GernError, match="32 x 256"):
+        gpu.Softmax(16384, rows_per_wave=4)
+
+
 def test_softmax_on_a_window_of_a_wider_buffer(gpu, oracle):
     # ld larger than ncol; columns outside the window stay as they were
     import torch
@@ -565,6 +616,37 @@ def test_qk_softmax_matches_oracle(gpu, oracle, M, N, D, max_keys, flags):
     # logits differ only by fp32 summation order
     assert np.max(np.abs(got - want) / want) < 1e-2
     assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-5)
+
+
+# More than sixteen column blocks per row: a wavefront collects the row's statistics in passes of sixteen
+# entries.  Widths that are whole passes, one block more, and a ragged last block; the exchange memory bounds
+# M x N (1024 rows at 65536 keys), and more is refused.
+@pytest.mark.parametrize("M,N,max_keys", [(520, 8192, 8192), (300, 4352, 8192), (257, 10000, 10240), (100, 16384, 16384),
+                                          (40, 65536, 65536)])
+def test_qk_softmax_tile_kernel_on_rows_wider_than_4096_keys(gpu, oracle, M, N, max_keys):
+    import torch
+    D = 64
+    qb, _ = oracle.to_bf16(oracle.normal((M, D), 50 + M))
+    kb, _ = oracle.to_bf16(oracle.normal((N, D), 60 + M))
+    scale = np.float32(1.0 / np.sqrt(D))
+    p = gpu.QKSoftmax(D, max_keys)
+    assert "view_score_tile" in p.source
+    S = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, scale)
+    torch.cuda.synchronize()
+    assert p.faults() == 0
+    got = S.cpu().numpy()
+    rows = sorted({0, 1, M // 2, M - 1, min(M - 1, 255), min(M - 1, 256)})
+    want = oracle.qk_softmax(qb[rows], kb, scale)
+    assert np.max(np.abs(got[rows] - want) / want) < 1e-2, (M, N)
+    assert not np.isnan(got).any()
+    assert np.all(np.abs(got.sum(axis=1, dtype=np.float64) - 1.0) < 1e-4)
+    if N == 65536:
+        big = torch.zeros((1025, D), dtype=torch.int16, device="cuda")
+        with pytest.raises(gpu.GernError, match="GERN_QK_SCRATCH_BYTES"):
+            p(big, _dev(kb.view(np.int16)), torch.zeros((1025, N), device="cuda"), scale)
+        with pytest.raises(gpu.GernError, match="4096"):
+            gpu.QKSoftmax(96, 8192)  # the row-block kernel keeps whole rows in registers
 
 
 def test_qk_softmax_tile_kernel_over_changing_shapes_and_scales(gpu, oracle):
