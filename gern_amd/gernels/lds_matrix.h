@@ -89,9 +89,11 @@ __device__ __forceinline__ RegTile4<H, W> allocate_static_vec() {
     return t;
 }
 
-// Pitch (in floats) of an LDS tile with W columns.
+// Pitch (in floats) of an LDS tile with W columns: rows that are a multiple of 16 floats long are padded by
+// four, so that rows 1, 2 or 4 apart (what the threads of a wavefront read when each holds a few rows of C)
+// do not start in the same bank, and 16-byte accesses stay aligned.
 constexpr int64_t lds_pitch(int64_t w) {
-    return (w % 32 == 0) ? w + 4 : w;
+    return (w % 16 == 0) ? w + 4 : w;
 }
 
 // An H x W tile in LDS (or a window of one): `owner` is the allocation to give
@@ -332,12 +334,46 @@ struct GlobalMatrix {
 
 // C(i, j) += sum_k A(i, k) * B(k, j), term by term in k order, on any of the
 // tile types above (gernels/mm/impl/matrix_multiply.h:63-76 of the reference).
+// The thread's elements of C are read once, updated in registers and written once per call: added to in
+// place, a C that lives in global memory would have to be stored after every term and the operands read
+// again after every store, because the compiler cannot rule out that the operands (generic pointers into
+// LDS) alias it.  (How much of that a compiler removes by itself differed between two versions of the
+// same compiler by a factor of 1.5 on the kernel_3 schedule.)
 template<int64_t k_dim, typename AT, typename BT, typename CT>
 __device__ __forceinline__ void matrix_multiply(const AT &A, const BT &B, CT &C) {
-    for (int64_t i = 0; i < AT::row; i++) {
-        for (int64_t j = 0; j < BT::col; j++) {
-            for (int64_t k = 0; k < k_dim; k++) {
-                C(i, j) += A(i, k) * B(k, j);
+    if constexpr (AT::row * BT::col <= 64) {
+        float c[AT::row][BT::col];
+#pragma unroll
+        for (int64_t i = 0; i < AT::row; i++) {
+#pragma unroll
+            for (int64_t j = 0; j < BT::col; j++) {
+                c[i][j] = C(i, j);
+            }
+        }
+#pragma unroll
+        for (int64_t i = 0; i < AT::row; i++) {
+#pragma unroll
+            for (int64_t j = 0; j < BT::col; j++) {
+                for (int64_t k = 0; k < k_dim; k++) {
+                    c[i][j] += A(i, k) * B(k, j);
+                }
+            }
+        }
+#pragma unroll
+        for (int64_t i = 0; i < AT::row; i++) {
+#pragma unroll
+            for (int64_t j = 0; j < BT::col; j++) {
+                C(i, j) = c[i][j];
+            }
+        }
+    } else {
+        for (int64_t i = 0; i < AT::row; i++) {
+            for (int64_t j = 0; j < BT::col; j++) {
+                float c = C(i, j);
+                for (int64_t k = 0; k < k_dim; k++) {
+                    c += A(i, k) * B(k, j);
+                }
+                C(i, j) = c;
             }
         }
     }
