@@ -365,7 +365,7 @@ def main():
                 "ms_per_step": head_t["wall_ms"],
                 "higher_is_better": True,
                 "scaling": "weak",
-                "vs_baseline": None,  # BASELINE.md publishes no number for this metric
+                "vs_baseline": None,  # the reference publishes no number for this metric
                 "dtype": "f32",
                 "data": "synthetic",
                 "config": {"workload": "three-stage fused separable blur chain (3-tap x, y, x; weights 1/3), 8192x8192 fp32 "
