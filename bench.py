@@ -296,7 +296,7 @@ def main():
     workloads = {}
     result = None
     # every workload is timed over at least MIN_SINGLE_LAUNCHES launches, whatever --steps says
-    steps2 = max(MIN_SINGLE_LAUNCHES, args.steps // 4)
+    steps2 = max(MIN_SINGLE_LAUNCHES, args.steps)  # launches of 0.4 ms and less: as many as the headline
     steps_gemm = max(MIN_SINGLE_LAUNCHES, args.steps // 10)
 
     def rotating(pairs, launch):
