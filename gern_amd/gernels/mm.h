@@ -436,7 +436,7 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
         const int k0 = kt * (int)kMfmaBK;
         const int64_t left_b = (((int64_t)B.rows - 1 - k0) * B.lda + B.cols) * 2;  // bytes from this stage's first row to the end
         const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(B.data + (int64_t)k0 * B.lda), 0, (int)(left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
+            (void *)(B.data + (int64_t)k0 * B.lda), 0, (int)(left_b < 0 ? 0 : left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
@@ -485,17 +485,33 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
     const int b_swz = (4 * (p / 4)) ^ (k16 ? 2 * (g & 1) : 0);  // (k & 3) == p / 4: the other terms are multiples of 4
     // Every LDS address below is ONE offset from the stage array: the compiler
     // tells the two stages apart only through short pointer chains.
-    auto load_a = [&](const unsigned char *stage, int tm, int s) {
+    // (LDS pointers in their own address space from the array on: every conversion to a generic pointer and
+    // back is a step in the chain along which the compiler keeps track of WHICH array an access goes to, and
+    // it follows only a few; an access it cannot place waits for all loads into the other stage)
+    typedef const __attribute__((address_space(3))) unsigned char *lds_bytes;
+    auto load_a = [&](const unsigned char *stage_generic, int tm, int s) {
+        lds_bytes stage = (lds_bytes)stage_generic;
         const int pos = ((k16 ? 4 : 2) * s + a_part) ^ a_swz;
         const int at = a_row_off + tm * kRows * 128 + pos * 16;
-        return *reinterpret_cast<const bf16x8_t *>(stage + at);
+        return *(const __attribute__((address_space(3))) bf16x8_t *)(stage + at);
     };
-    auto load_b = [&](const unsigned char *stage, int tn, int s) {
+    // The lane's own part of a B fragment's address is ONE value per column tile that the compiler may not
+    // take apart (it would spread the sum over a chain of pointer steps, and lose track of the array at the
+    // end of a long one): array + that value + a constant.
+    int b_lane[TN];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
         const int chunk = ((b_col0 + tn * kRows) / 8 + (p % 4) / 2) ^ b_swz;
-        const int at = A_BYTES + ((k16 ? 32 : 16) * s + b_krow) * 512 + chunk * 16 + (p % 2) * 8;
-        const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + at));
+        int v = b_krow * 512 + chunk * 16 + (p % 2) * 8;
+        asm volatile("" : "+v"(v));
+        b_lane[tn] = v;
+    }
+    auto load_b = [&](const unsigned char *stage_generic, int tn, int s) {
+        lds_bytes lane_base = (lds_bytes)stage_generic + b_lane[tn];
+        const int at = A_BYTES + (k16 ? 32 : 16) * s * 512;
+        const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(lane_base + at));
         const v4s_t hi =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(stage + (at + 4 * 512)));
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t *)(lane_base + (at + 4 * 512)));
         const v8s_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return __builtin_bit_cast(bf16x8_t, both);
     };
@@ -539,6 +555,25 @@ __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, t
                     }
                 }
             }
+            // THE ORDER OF ISSUE IS WRITTEN OUT (sched_group_barrier: the next n instructions of a kind).
+            // Left to itself the compiler reads a fragment just before its first use -- eight matrix
+            // instructions, two reads, a wait for them, eight more -- and what a wavefront loses to LDS latency
+            // the other wavefront of the SIMD only partly makes up (4096^3: 105.6 -> 101.4 us, 108.1 -> 103.4 us
+            // on a slower GPU).  Here: the twelve reads of the first phase; then, phase by phase, the reads of
+            // the NEXT phase spread among the sixteen matrix instructions of this one.
+            static_assert(HALF == 4 && TN == 4 && KSTEPS == 2, "the order of issue below is written out for these");
+#define GERN_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define GERN_READ_THEN(n) GERN_SGB(0x100, 1); GERN_SGB(0x008, n)
+            GERN_SGB(0x100, 12);
+            GERN_READ_THEN(4); GERN_READ_THEN(4); GERN_READ_THEN(4); GERN_READ_THEN(4);
+            GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1);
+            GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1);
+            GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1); GERN_READ_THEN(1);
+            GERN_SGB(0x008, 4);
+            GERN_READ_THEN(4); GERN_READ_THEN(4); GERN_READ_THEN(4); GERN_READ_THEN(4);
+            GERN_SGB(0x008, 16);
+#undef GERN_READ_THEN
+#undef GERN_SGB
         } else {
             bf16x8_t af[2][TM], bfr[2][TN];
 #pragma unroll
