@@ -347,18 +347,22 @@ namespace detail {
 // stage 167; two wavefront groups half a stage out of phase (one computing
 // while the other moves data) 140; this one, with 64-bit lane addresses, 131;
 // on v_mfma_f32_32x32x16_bf16 (MfmaAcc) 116-120; on v_mfma_f32_16x16x32_bf16
-// (MfmaAcc16) 104-109.
+// (MfmaAcc16) 104-109, with its order of issue written out 101-106.
 //
-// THE KERNEL IS BOUND BY POWER, not by issue slots: the two instructions need
-// the same number of cycles (246 500 and 250 800 per launch and XCD, counted by
+// THE KERNEL RUNS INTO THE POWER LIMIT: the two instructions need the same
+// number of cycles (246 500 and 250 800 per launch and XCD, counted by
 // GRBM_GUI_ACTIVE), but the clock settles at 2.05 GHz with the first and at
-// 2.28 GHz with the second, and the time follows the clock.  Variants that
-// change the schedule and not the work leave the time where it is: the K loop
-// rotated so that the barrier stands before a stage's last sixteen
-// instructions (they cover the wait for the next stage's first fragments)
-// takes 4 % MORE cycles at a 3 % higher clock; C stored in whole 128-byte
-// lines (lanes p and p ^ 8 swapping a piece through DPP) instead of 64-byte
-// halves: no difference.
+// 2.28-2.35 GHz with the second, and the time follows the clock.  Close to
+// the clock's ceiling cycles count again: with the order of issue inside a
+// stage written out (compute(), below) the 16 x 16 x 32 kernel takes 221 100
+// cycles at 2.18 GHz, 101.3 us.  What did not help, each measured against the
+// kernel as it is in one process: the K loop rotated so that the barrier
+// stands before a stage's last sixteen instructions (they cover the wait for
+// the next stage's first fragments), with the compiler's order or a written-out
+// one (+2 to +3 %); the loads of the next stage spread among the first phase's
+// matrix instructions instead of issued in front of them (+1 %); C stored in
+// whole 128-byte lines (lanes p and p ^ 8 swapping a piece through DPP)
+// instead of 64-byte halves (no difference).
 template<int64_t BM, int64_t BN, int64_t KC, typename Acc>
 __device__ __forceinline__ void mfma_direct(const GlobalView<BM, KC, uint16_t, true> &A,
                                             const GlobalView<KC, BN, uint16_t, true> &B, Acc &C) {
