@@ -103,5 +103,64 @@ protected:
     Variable k{"k"};
 };
 
+// A data structure without index fields: one float.
+class ScalarCPU : public TableADT {
+public:
+    ScalarCPU(const std::string &name = "scalar")
+        : TableADT(name, "gern::impl::ScalarCPU") {
+        allocate_call = call("gern::impl::ScalarCPU::allocate");
+        query_call = call("open");
+    }
+};
+
+// *output = input[0]: consumes the array's first element, produces the whole (field-less) scalar.
+class first_element : public AbstractFunction {
+public:
+    first_element()
+        : input(new const ArrayCPU("input")), output(new const ScalarCPU("output")) {
+    }
+    Annotation getAnnotation() override {
+        Variable one("one");
+        return annotate(Computes(Produces::Subset(output, {}), Consumes::Subsets(SubsetObjMany{SubsetObj(input, {Expr(0), Expr(1)})})));
+    }
+    std::vector<std::string> getHeader() override {
+        return {"array_host.h"};
+    }
+    FunctionSignature getFunction() override {
+        FunctionSignature f;
+        f.name = "gern::impl::first_element";
+        f.args = {Parameter(input), Parameter(output)};
+        return f;
+    }
+
+protected:
+    AbstractDataTypePtr input, output;
+};
+
+// output[x .. x+step) = input[x .. x+step) + *scalar
+class add_scalar : public AbstractFunction {
+public:
+    add_scalar()
+        : input(new const ArrayCPU("input")), scalar(new const ScalarCPU("scalar")), output(new const ArrayCPU("output")) {
+    }
+    Annotation getAnnotation() override {
+        Variable x("x"), step("step");
+        return annotate(Tileable(x = Expr(0), output["size"], step, Produces::Subset(output, {x, step}),
+                                 Consumes::Subsets(SubsetObjMany{SubsetObj(input, {x, step}), SubsetObj(scalar, {})})));
+    }
+    std::vector<std::string> getHeader() override {
+        return {"array_host.h"};
+    }
+    FunctionSignature getFunction() override {
+        FunctionSignature f;
+        f.name = "gern::impl::add_scalar";
+        f.args = {Parameter(input), Parameter(scalar), Parameter(output)};
+        return f;
+    }
+
+protected:
+    AbstractDataTypePtr input, scalar, output;
+};
+
 }  // namespace annot
 }  // namespace gern

@@ -83,5 +83,33 @@ inline void reduction(ArrayCPU in, ArrayCPU out, int64_t k) {
     }
 }
 
+// One float that a program computes once and every tile reads: a data
+// structure without index fields (its query, open(), takes nothing).
+struct ScalarCPU {
+    float *value = nullptr;
+    static ScalarCPU allocate() {
+        ScalarCPU s;
+        s.value = static_cast<float *>(std::calloc(1, sizeof(float)));
+        return s;
+    }
+    ScalarCPU open() const {
+        return *this;
+    }
+    void destroy() {
+        std::free(value);
+        value = nullptr;
+    }
+};
+
+// *out = in[0] (what the array starts with)
+inline void first_element(ArrayCPU in, ScalarCPU out) {
+    *out.value = in.data[0];
+}
+
+// out[i] = in[i] + *s
+inline void add_scalar(ArrayCPU in, ScalarCPU s, ArrayCPU out) {
+    detail::add_constant(in, out, in.size, *s.value);
+}
+
 }  // namespace impl
 }  // namespace gern

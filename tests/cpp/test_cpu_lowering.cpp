@@ -578,4 +578,31 @@ CASE("mm.function_ptr_with_bound_tiles") {  // test-cpu-mm.cpp:189-264
     }
 }
 
+// A query that takes nothing is moved to the top of the generated function when it opens a PARAMETER (its
+// latency then hides behind what follows); a data structure that the program itself allocates and computes
+// must be opened behind the statements that define it.
+CASE("array.fieldless_query_of_an_intermediate_stays_behind_its_definition") {
+    auto in = arrayDS("input_con"), out = arrayDS("output_con");
+    auto s = AbstractDataTypePtr(new const annot::ScalarCPU("first"));
+    annot::first_element first_element;
+    annot::add_scalar add_scalar;
+    Variable step("step");
+    Runner run(Composable({first_element(in, s), Tile(out["size"], step)(add_scalar(in, s, out))}));
+    REQUIRE_NOTHROW(run.compile(hostOptions()));
+    const std::string src = run.getSource();
+    const size_t allocated = src.find("ScalarCPU::allocate"), computed = src.find("first_element("), opened = src.find(".open(");
+    REQUIRE(allocated != std::string::npos);
+    REQUIRE(computed != std::string::npos);
+    REQUIRE(opened != std::string::npos);
+    REQUIRE(allocated < computed);
+    REQUIRE(computed < opened);
+    Arrays t(10);
+    for (int64_t i = 0; i < t.a.size; i++) {
+        t.a.data[i] = (float)(i + 5);
+    }
+    int64_t step_val = 5;
+    REQUIRE_NOTHROW(run.evaluate({{in.getName(), &t.a}, {out.getName(), &t.b}, {step.getName(), &step_val}}));
+    t.expect_offset(5);  // every element grew by the first one
+}
+
 CHECK_MAIN()
