@@ -52,12 +52,16 @@ def test_softmax_random_widths_and_rows(gpu, oracle):
     import torch
     rng = np.random.RandomState(102)
     widths = [int(rng.randint(1, 3000)) for _ in range(6)] + [512, 1024, 1280, 1536, 2048, 2560, 3072, 5120, 7168, 8192]
+    # rows wider than one wavefront holds: cut into 4, 8 or 16 pieces, evenly or not
+    widths += [int(rng.randint(8193, 16385)), int(rng.randint(16385, 32769)), int(rng.randint(32769, 65537)), 24576]
     for case, ncol in enumerate(widths):
         rows = int(rng.randint(1, 70))
         per_wave_chunks = 32
         rpw = int(rng.choice([1, 1, 2, 3]))
         chunks = (ncol + 255) // 256
         if rpw * chunks > per_wave_chunks and not (ncol >= 1024 and ncol % 512 == 0):
+            rpw = 1
+        if ncol > 8192:
             rpw = 1
         x = oracle.normal((rows, ncol), 300 + case, 0.0, 3.0)
         sm = gpu.Softmax(ncol, rows_per_wave=rpw)
