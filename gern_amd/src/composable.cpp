@@ -279,9 +279,15 @@ void Computation::init_annotation() {
             if (intermediates.count(input.getDS().getName())) {
                 continue;
             }
+            // One substitution per stage between this input and the output: the fields end up over the
+            // variables of the LAST stage, which are the ones a tile or a stage around the chain renames.
             std::vector<Expr> fields;
             for (const auto &f : input.getFields()) {
-                fields.push_back(substitute(f, defs));
+                Expr over_output = f;
+                for (size_t stage = 0; stage < composed.size(); stage++) {
+                    over_output = substitute(over_output, defs);
+                }
+                fields.push_back(over_output);
             }
             true_inputs.push_back(SubsetObj(input.getDS(), fields));
         }

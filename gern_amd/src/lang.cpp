@@ -1117,7 +1117,9 @@ Annotation refreshVariables(Annotation annot, std::map<Variable, Variable> &new_
 
     Substitution s;
     for (const auto &v : getVariables(annot)) {
-        if (keep.count(v.getName())) {
+        // So does a variable the user has bound to a value: it is a constant wherever it appears, and the
+        // footprint of a tile or a stage around the body may need it (a halo of stride - 1 elements).
+        if (keep.count(v.getName()) || v.isBound()) {
             continue;
         }
         Variable fresh(getUniqueName(v.getName()), v.getDatatype(), v.isConstExpr());

@@ -20,6 +20,7 @@
 #include "library/device_host.h"
 #include "library/matrix_device_annot.h"
 
+#include "annot/blur.h"
 #include "annot/lds_matrix.h"
 #include "annot/reduce.h"
 
@@ -817,6 +818,87 @@ static bool buildWithPrefix(Runner &run, Composable program, const Runner::Optio
     run.compile(o);
     last_source = run.getSource();
     return true;
+}
+
+CASE("schedule.blur_chain_on_halo_tiles_staged_into_lds") {
+    // A three-stage blur (x, y, x; the chain of apps/blur/blur.cpp:31-73) as a schedule at the level of the API:
+    // every workgroup stages its input tile INTO LDS WITH THE HALO that the composed annotations infer
+    // (16 x 64 outputs need 18 x 68 inputs), every thread takes the 4 x 8 window of it that its own 2 x 4
+    // outputs need, and the two intermediates are register tiles of the thread (4 x 6, then 2 x 6).
+    constexpr int64_t rows = 128, cols = 128, in_rows = rows + 2, in_cols = cols + 4;
+    using InType = annot::MatrixGlobalToShared<in_rows, in_cols>;
+    using OutType = annot::MatrixGlobalToGlobal<rows, cols>;
+    using TempType = annot::MatrixQueryRegNoVector<in_rows, in_cols>;
+    auto input = AbstractDataTypePtr(new const InType("input", false));
+    auto output = AbstractDataTypePtr(new const OutType("output", false));
+    auto t1 = AbstractDataTypePtr(new const TempType("t1", true));
+    auto t2 = AbstractDataTypePtr(new const TempType("t2", true));
+    InType view_of("input_view", false);
+    Variable stride("stride"), block_r("block_r"), block_c("block_c"), thread_r("thread_r"), thread_c("thread_c"), smem_size("smem_size");
+    std::map<std::string, Variable> three{{"stride", stride.bind(3)}};
+    annot::BlurXPerThread first{input, t1};
+    annot::BlurYPerThread second{t1, t2};
+    annot::BlurXPerThread third{t2, output};
+    Composable chain(new const Computation({first[three](input, t1), second[three](t1, t2), third[three](t2, output)}));
+    Composable program = Global(
+        (Tile(output["row"], block_r.bind(16)) || Grid::Unit::BLOCK_Y)((Tile(output["col"], block_c.bind(64)) || Grid::Unit::BLOCK_X)(
+            Stage(input, (Tile(output["row"], thread_r.bind(2)) || Grid::Unit::THREAD_Y)((Tile(output["col"], thread_c.bind(4)) || Grid::Unit::THREAD_X)(
+                             Stage(input, view_of.getView(), chain)))))),
+        {}, smem_size, LdsManager(smem_size));
+    Runner run(program);
+    const bool ran = build(run, program);
+    // the staged tile and the thread's window carry the inferred halo: (rows + 2) x (cols + 4)
+    REQUIRE(last_source.find("stage_into_smem<((block_r + stride) - 1), ((((block_c + stride) - 1) + stride) - 1)>") != std::string::npos);
+    REQUIRE(last_source.find("get_view<((thread_r + stride) - 1), ((((thread_c + stride) - 1) + stride) - 1)>") != std::string::npos);
+    REQUIRE(last_source.find("blur_y_per_thread") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    impl::MatrixGPU in(in_rows, in_cols, in_cols), out(rows, cols, cols);
+    std::vector<float> h(in_rows * in_cols);
+    for (int64_t e = 0; e < in_rows * in_cols; e++) {
+        h[e] = (float)((e * 37 + (e / in_cols) * 11) % 97) * 0.25f - 7.0f;
+    }
+    impl::hipCheck(gern_hip_memcpy_h2d(in.data, h.data(), sizeof(float) * h.size()));
+    hip::GlobalMatrixF32 pin{in.data}, pout{out.data};
+    int64_t smem = 18 * 72 * 4 + 1024;
+    run.evaluate({{"input", &pin}, {"output", &pout}, {smem_size.getName(), &smem}});
+    REQUIRE_EQ(run.ldsOverflows(), (int64_t)0);
+    // the stages one after the other on the host, same order of additions, same division
+    std::vector<float> a(in_rows * (in_cols - 2)), b(rows * (in_cols - 2)), want(rows * cols);
+    for (int64_t i = 0; i < in_rows; i++) {
+        for (int64_t j = 0; j < in_cols - 2; j++) {
+            float sum = 0.0f;
+            for (int64_t t = 0; t < 3; t++) {
+                sum += h[i * in_cols + j + t];
+            }
+            a[i * (in_cols - 2) + j] = sum / 3.0f;
+        }
+    }
+    for (int64_t i = 0; i < rows; i++) {
+        for (int64_t j = 0; j < in_cols - 2; j++) {
+            float sum = 0.0f;
+            for (int64_t t = 0; t < 3; t++) {
+                sum += a[(i + t) * (in_cols - 2) + j];
+            }
+            b[i * (in_cols - 2) + j] = sum / 3.0f;
+        }
+    }
+    for (int64_t i = 0; i < rows; i++) {
+        for (int64_t j = 0; j < cols; j++) {
+            float sum = 0.0f;
+            for (int64_t t = 0; t < 3; t++) {
+                sum += b[i * (in_cols - 2) + j + t];
+            }
+            want[i * cols + j] = sum / 3.0f;
+        }
+    }
+    std::vector<float> got = out.get();
+    for (int64_t e = 0; e < rows * cols; e++) {
+        REQUIRE_EQ(got[e], want[e]);
+    }
+    in.destroy();
+    out.destroy();
 }
 
 CASE("function_ptr.device_function_called_from_a_kernel") {
