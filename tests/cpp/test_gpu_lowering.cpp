@@ -787,6 +787,104 @@ CASE("schedule.gemm_float4_register_tiles") {  // gernels/mm/mm_registers.cu:13-
     check_schedule_product<m, n, k>(run);
 }
 
+// One output element per thread, operands and result windows of the matrices in global memory: the
+// schedules of gernels/mm/kernel_1.cu:13-64 (rows on x) and kernel_2.cu:13-65 (columns on x, so that the
+// lanes of a wavefront read consecutive elements of B and write consecutive elements of C).
+static void element_per_thread_schedule(bool columns_on_x) {
+    constexpr int64_t m = 64, n = 64, k = 64;
+    using AType = annot::MatrixGlobalToGlobal<m, k>;
+    using BType = annot::MatrixGlobalToGlobal<k, n>;
+    using CType = annot::MatrixGlobalToGlobal<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    Variable k_dim("k_dim"), block_x("block_x"), block_y("block_y"), thread_x("thread_x"), thread_y("thread_y");
+    block_x = block_x.bind(32);
+    block_y = block_y.bind(32);
+    thread_x = thread_x.bind(1);
+    thread_y = thread_y.bind(1);
+    k_dim = k_dim.bind(k);
+    annot::MatrixMultiplyScalar mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    const Grid::Unit rows_on_blocks = columns_on_x ? Grid::Unit::BLOCK_Y : Grid::Unit::BLOCK_X;
+    const Grid::Unit cols_on_blocks = columns_on_x ? Grid::Unit::BLOCK_X : Grid::Unit::BLOCK_Y;
+    const Grid::Unit rows_on_threads = columns_on_x ? Grid::Unit::THREAD_Y : Grid::Unit::THREAD_X;
+    const Grid::Unit cols_on_threads = columns_on_x ? Grid::Unit::THREAD_X : Grid::Unit::THREAD_Y;
+    Composable program = Global((Tile(C["row"], block_x) || rows_on_blocks)((Tile(C["col"], block_y) || cols_on_blocks)(
+        (Tile(C["row"], thread_x) || rows_on_threads)((Tile(C["col"], thread_y) || cols_on_threads)(mm_sp(A, B, C))))));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("query_global_2_global<thread_x, thread_y>") != std::string::npos);
+    REQUIRE(last_source.find("__launch_bounds__(1024)") != std::string::npos);  // 32 x 32 threads
+    // which index of the thread walks the columns of C
+    const std::string col_index = columns_on_x ? "threadIdx.x" : "threadIdx.y";
+    REQUIRE(last_source.find("((" + col_index + " / 1) % (((thread_y + (block_y - 0)) - 1) / thread_y))") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    check_schedule_product<m, n, k>(run);
+}
+
+CASE("schedule.gemm_one_element_per_thread") {  // gernels/mm/kernel_1.cu:13-92 of the reference
+    element_per_thread_schedule(false);
+}
+
+CASE("schedule.gemm_one_element_per_thread_columns_on_x") {  // gernels/mm/kernel_2.cu:13-93 of the reference
+    element_per_thread_schedule(true);
+}
+
+CASE("schedule.gemm_whole_product_in_one_call") {  // gernels/mm/mm_trivial.cu:13-78 of the reference
+    // No tiling at all: one thread multiplies the whole matrices where they lie.
+    constexpr int64_t m = 8, n = 8, k = 8;
+    using AType = annot::MatrixQueryRegNoVector<m, k>;
+    using BType = annot::MatrixQueryRegNoVector<k, n>;
+    using CType = annot::MatrixQueryRegNoVector<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    Variable k_dim("k_dim");
+    annot::MatrixMultiplyScalar mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim.bind(k)}}];
+    Composable program = Global(mm_sp(A, B, C));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("gernels::matrix_multiply<k_dim>") != std::string::npos);
+    REQUIRE(last_source.find("__launch_bounds__(1)") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    check_schedule_product<m, n, k>(run);
+}
+
+CASE("schedule.gemm_register_tiles_rows_on_threads") {  // gernels/mm/mm_shared.cu:13-97 of the reference
+    // 2 x 8 tiles of C on the threads of one workgroup, each a register copy that is multiplied into over
+    // one K tile and written back (the reference's file is named for LDS and stages nothing into it).
+    constexpr int64_t m = 8, n = 8, k = 8;
+    using AType = annot::MatrixGPUVec<m, k>;
+    using BType = annot::MatrixGPUVec<k, n>;
+    using CType = annot::MatrixGPUVec<m, n>;
+    auto A = AbstractDataTypePtr(new const AType("A", false));
+    auto B = AbstractDataTypePtr(new const BType("B", false));
+    auto C = AbstractDataTypePtr(new const CType("C", false));
+    Variable k_dim("k_dim"), c_row("c_row"), c_col("c_col"), k_tile("k_tile");
+    c_row = c_row.bind(2);
+    c_col = c_col.bind(8);
+    k_tile = k_tile.bind(8);
+    k_dim = k_dim.bind(k);
+    annot::MatrixMultiplyReg mm(A, B, C);
+    auto &mm_sp = mm[{{"k_dim", k_dim}}];
+    Composable program = Global((Tile(C["row"], c_row) || Grid::Unit::THREAD_X)(
+        (Tile(C["col"], c_col) || Grid::Unit::THREAD_Y)(Reduce(k_dim, k_tile)(mm_sp(A, B, C)))));
+    Runner run(program);
+    const bool ran = build(run, program);
+    REQUIRE(last_source.find("matrix_multiply_reg") != std::string::npos);
+    REQUIRE(last_source.find("query<c_row, k_tile>") != std::string::npos);
+    if (!ran) {
+        return;
+    }
+    check_schedule_product<m, n, k>(run);
+}
+
 // ---- FunctionPtr on the device -----------------------------------------------------------------
 
 static Runner::Options deviceFunctionOptions(const std::string &file) {
