@@ -975,38 +975,51 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
         __builtin_amdgcn_make_buffer_rsrc((void *)A.data, 0, (int)((((int64_t)A.rows - 1) * A.lda + A.cols) * 4), kRawBuffer);
     const int row_bytes_b = (int)B.lda * 4;
     // Wavefront w issues A instructions 4w .. 4w+3 (8 rows each) and B
-    // instructions 4w .. 4w+3 (one K row each) of every stage.
-    auto issue_from = [&](int kt, unsigned char *dst, const int (&off_a)[4]) {
+    // instructions 4w .. 4w+3 (one K row each) of every stage.  What a stage's
+    // loads need is computed apart from the loads themselves (Loads), so that
+    // the arithmetic can stand before the barrier that the loads follow.
+    // The lanes' A offsets for a partial last stage: chunks past K are sent out of range.
+    int lane_off_a_tail[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int row = 8 * (wu * 4 + j) + lane / 8;
+        const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+        lane_off_a_tail[j] = (tail == 0 || chunk * 4 < tail) ? lane_off_a[j] : kOutOfRange;
+    }
+    struct Loads {
+        __amdgpu_buffer_rsrc_t desc_b;
+        int k0_bytes;
+        int off_a[4];
+    };
+    auto prepare = [&](int kt) {
+        Loads l;
         const int k0 = kt * BK;
-        const int64_t left_b = (((int64_t)B.rows - 1 - k0) * B.lda + B.cols) * 4;
-        const __amdgpu_buffer_rsrc_t desc_b = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(B.data + (int64_t)k0 * B.lda), 0, (int)(left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
+        const int64_t left_b = k0 < (int64_t)B.rows ? (((int64_t)B.rows - 1 - k0) * B.lda + B.cols) * 4 : 0;  // 0: all zeros
+        l.desc_b = __builtin_amdgcn_make_buffer_rsrc((void *)(B.data + (int64_t)k0 * B.lda), 0,
+                                                     (int)(left_b < 0xFFFFFFFFll ? left_b : 0xFFFFFFFFll), kRawBuffer);
+        l.k0_bytes = k0 * 4;
+        // workgroup-uniform, and selects rather than branches, so that a stage stays one block of code; a stage
+        // past K (the loop below takes stages in pairs) is filled with zeros: every lane out of range
+        const bool partial = tail != 0 && kt == nk - 1;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            l.off_a[j] = kt >= nk ? kOutOfRange : partial ? lane_off_a_tail[j] : lane_off_a[j];
+        }
+        return l;
+    };
+    auto issue = [&](const Loads &l, unsigned char *dst) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_a, (__attribute__((address_space(3))) void *)(dst + (i * 1024)), 16,
-                                                     off_a[j], k0 * 4, 0, 0);
+                                                     l.off_a[j], l.k0_bytes, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int i = wu * 4 + j;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(desc_b,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(l.desc_b,
                                                      (__attribute__((address_space(3))) void *)(dst + (A_BYTES + i * 1024)),
                                                      16, lane_off_b, i * row_bytes_b, 0, 0);
-        }
-    };
-    auto issue = [&](int kt, unsigned char *dst) {
-        if (tail != 0 && kt == nk - 1) {  // workgroup-uniform; at most once per call
-            int off_tail[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int row = 8 * (wu * 4 + j) + lane / 8;
-                const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-                off_tail[j] = chunk * 4 < tail ? lane_off_a[j] : kOutOfRange;
-            }
-            issue_from(kt, dst, off_tail);
-        } else {
-            issue_from(kt, dst, lane_off_a);
         }
     };
 
@@ -1014,28 +1027,28 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
     const int a_row = (w / Acc::WC) * 64 + (lane % 32);
     const int a_swz = ((lane % 32) >> 1) & 7;  // rows 64 wr + 32 tm + lane % 32: the other terms are multiples of 16
     const int b_off = A_BYTES + (4 * half) * 1024 + ((w % Acc::WC) * 128 + 4 * (lane % 32)) * 4;
-    auto compute = [&](const unsigned char *stage) {
+    // The fragments of K block kb (8 deep) of a stage: two reads for A, four for B.
+    auto read_block = [&](const unsigned char *stage, int kb, f32x4_native (&a)[Acc::TM], f32x4_native (&b)[4]) {
 #pragma unroll
-        for (int kb = 0; kb < BK / 8; kb++) {
-            f32x4_native a[Acc::TM], b[4];
+        for (int tm = 0; tm < Acc::TM; tm++) {
+            const int at = (a_row + tm * 32) * 128 + (((2 * kb + half) ^ a_swz) * 16);
+            a[tm] = *reinterpret_cast<const f32x4_native *>(stage + at);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int at = b_off + (8 * kb + j) * 1024;
+            b[j] = *reinterpret_cast<const f32x4_native *>(stage + at);
+        }
+    };
+    // and their 32 matrix instructions (64 cycles each)
+    auto multiply_block = [&](const f32x4_native (&a)[Acc::TM], const f32x4_native (&b)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
 #pragma unroll
             for (int tm = 0; tm < Acc::TM; tm++) {
-                const int at = (a_row + tm * 32) * 128 + (((2 * kb + half) ^ a_swz) * 16);
-                a[tm] = *reinterpret_cast<const f32x4_native *>(stage + at);
-            }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int at = b_off + (8 * kb + j) * 1024;
-                b[j] = *reinterpret_cast<const f32x4_native *>(stage + at);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-#pragma unroll
-                for (int tm = 0; tm < Acc::TM; tm++) {
-#pragma unroll
-                    for (int tn = 0; tn < Acc::TN; tn++) {
-                        C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][j], b[j][tn], C.acc[tm][tn], 0, 0, 0);
-                    }
+                for (int tn = 0; tn < Acc::TN; tn++) {
+                    C.acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][j], b[j][tn], C.acc[tm][tn], 0, 0, 0);
                 }
             }
         }
@@ -1045,22 +1058,65 @@ __device__ __forceinline__ void mfma_direct_f32(const GlobalView<BM, KC, float, 
         __builtin_amdgcn_s_barrier();
     };
 
-    issue(0, stage_even_f32);
-    arrive();
-    for (int kt = 0; kt < nk; kt += 2) {
-        if (kt + 1 < nk) {
-            issue(kt + 1, stage_odd_f32);
-        }
-        compute(stage_even_f32);
+    // A stage is four K blocks, and the fragments of a block are read WHILE THE BLOCK BEFORE IT IS MULTIPLIED
+    // (two sets of fragment registers, p and q).  The stage's one barrier stands before its last block: by then
+    // every wavefront holds that block's fragments in registers, so the stage's LDS can be given to the loads of
+    // the stage after the next, and the first block of the next stage (whose loads were issued a stage ago) is
+    // read behind the barrier, under the 32 matrix instructions of the last block.  Left to the compiler's
+    // order, every block began with its own reads and a wait for them, four times per stage and on both
+    // wavefronts of a SIMD at once (they leave the barrier together): 8.5 % of the launch without a matrix
+    // instruction in flight; about 5 % now.  The order is written out with sched_group_barrier (0x008 matrix
+    // instruction, 0x100 LDS read, 0x010 memory instruction), one region per side of the barrier; the
+    // arithmetic for the loads (prepare) stands in the region before the barrier.  Measured, 4096^3, same
+    // process, alternating (us per launch; the order the compiler chose before: 952): a block's six reads one
+    // matrix instruction apart, two apart or back to back 921-924, five apart (spread over the block) 930; the
+    // eight loads three or two matrix instructions apart 918-919, in pairs 923, back to back 929-936, the
+    // four loads of B moved into the next stage's first block 930 against 925.  Without the loads the loop
+    // takes 901-909, without the barrier 4 us less: what is left is what the loads and reads cost in issue.
+    f32x4_native ap[Acc::TM], bp[4], aq[Acc::TM], bq[4];
+#define GERN_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define GERN_SIX_READS_EVERY(n) \
+    GERN_SGB(0x100, 1); GERN_SGB(0x008, n); GERN_SGB(0x100, 1); GERN_SGB(0x008, n); GERN_SGB(0x100, 1); GERN_SGB(0x008, n); \
+    GERN_SGB(0x100, 1); GERN_SGB(0x008, n); GERN_SGB(0x100, 1); GERN_SGB(0x008, n); GERN_SGB(0x100, 1); GERN_SGB(0x008, n)
+#define GERN_EIGHT_LOADS_EVERY(n) \
+    GERN_SGB(0x010, 1); GERN_SGB(0x008, n); GERN_SGB(0x010, 1); GERN_SGB(0x008, n); GERN_SGB(0x010, 1); GERN_SGB(0x008, n); \
+    GERN_SGB(0x010, 1); GERN_SGB(0x008, n); GERN_SGB(0x010, 1); GERN_SGB(0x008, n); GERN_SGB(0x010, 1); GERN_SGB(0x008, n); \
+    GERN_SGB(0x010, 1); GERN_SGB(0x008, n); GERN_SGB(0x010, 1); GERN_SGB(0x008, n)
+    // On entry p holds block 0 of `cur`; on exit, block 0 of `nxt`.  Stage kt + 2 is loaded into `cur`.
+    auto stage = [&](unsigned char *cur, const unsigned char *nxt, int kt) {
+        const Loads after_next = prepare(kt + 2);
+        read_block(cur, 1, aq, bq);
+        multiply_block(ap, bp);
+        read_block(cur, 2, ap, bp);
+        multiply_block(aq, bq);
+        read_block(cur, 3, aq, bq);
+        multiply_block(ap, bp);
+        GERN_SGB(0x008, 2); GERN_SIX_READS_EVERY(2); GERN_SGB(0x008, 18);
+        GERN_SGB(0x008, 2); GERN_SIX_READS_EVERY(2); GERN_SGB(0x008, 18);
+        GERN_SGB(0x008, 2); GERN_SIX_READS_EVERY(2); GERN_SGB(0x008, 18);
+        __builtin_amdgcn_sched_barrier(0);
         arrive();
-        if (kt + 1 < nk) {
-            if (kt + 2 < nk) {
-                issue(kt + 2, stage_even_f32);
-            }
-            compute(stage_odd_f32);
-            arrive();
-        }
+        read_block(nxt, 0, ap, bp);
+        issue(after_next, cur);
+        multiply_block(aq, bq);
+        GERN_SGB(0x008, 1); GERN_SIX_READS_EVERY(1); GERN_EIGHT_LOADS_EVERY(3); GERN_SGB(0x008, 1);
+    };
+#undef GERN_EIGHT_LOADS_EVERY
+#undef GERN_SIX_READS_EVERY
+#undef GERN_SGB
+
+    // Stages are taken in pairs, one per LDS array, in a loop without a branch inside: when the number of
+    // stages is odd the last pair's second stage is all zeros (its loads are sent out of range, above), and
+    // the loads and reads that the last stages issue for stages past K fetch nothing and feed nothing.
+    issue(prepare(0), stage_even_f32);
+    arrive();
+    issue(prepare(1), stage_odd_f32);
+    read_block(stage_even_f32, 0, ap, bp);
+    for (int kt = 0; kt < nk; kt += 2) {
+        stage(stage_even_f32, stage_odd_f32, kt);
+        stage(stage_odd_f32, stage_even_f32, kt + 1);
     }
+    arrive();  // no load into LDS is in flight when the next call begins
 }
 
 }  // namespace detail
