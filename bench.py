@@ -455,44 +455,47 @@ def main():
         steps_here = steps_gemm if variant == "f32" else max(steps_gemm, args.steps)
         t = measure(lambda: g(dA, dB, dC), 5, steps_here, torch, gern_amd)
         vendor = {}
+        # The vendor library on the same operands, for comparison (not part of the product).  bf16: torch.mm with
+        # fp32 output is the same contract (bf16 in, fp32 accumulate, fp32 C); with bf16 output the library writes
+        # half the bytes.  fp32: torch.mm (TF32 is off by default).  This build's kernel and the library's are
+        # timed in turn, twice, each time with the same warm-up, and every kernel keeps its better turn: on a GPU
+        # whose clock follows its power draw and temperature, whichever runs second would otherwise pay for the first.
         if variant == "bf16":
-            # The vendor library on the same operands, for comparison (not part of the product): torch.mm with fp32
-            # output is the same contract (bf16 in, fp32 accumulate, fp32 C); with bf16 output the library writes
-            # half the bytes.  This build's kernel and the library's are timed in turn, twice, each time with the
-            # same warm-up, and every kernel keeps its better turn: on a GPU whose clock follows its power draw
-            # and temperature, whichever runs second would otherwise pay for the first.
             tA, tB = dA.view(torch.bfloat16), dB.view(torch.bfloat16)
             out_bf16 = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
             calls = {"gemm_bf16_4096_vendor": lambda: torch.mm(tA, tB, out_dtype=torch.float32, out=dC),
                      "gemm_bf16_4096_vendor_bf16_out": lambda: torch.mm(tA, tB, out=out_bf16)}
-            turns = {"ours": [t]}
-            for turn in range(2):
-                for name, call in calls.items():
-                    try:
-                        turns.setdefault(name, []).append(measure(call, 5, steps_here, torch, gern_amd))
-                    except Exception as e:  # a torch without out_dtype: say so, do not fail the benchmark
-                        vendor[name] = {"error": str(e)[:200]}
-                if turn == 0:
-                    turns["ours"].append(measure(lambda: g(dA, dB, dC), 5, steps_here, torch, gern_amd))
-            t = min(turns["ours"], key=lambda x: x["ms"])
-            for name in calls:
-                if name in turns:
-                    tv = min(turns[name], key=lambda x: x["ms"])
-                    tfv = 2.0 * n ** 3 / (tv["ms"] * 1e-3) / 1e12
-                    vendor[name] = {"TFLOP/s": tfv, "ms": tv["ms"], "ms_median": tv["ms_median"], "ms_min": tv["ms_min"],
-                                    "ms_turns": [x["ms"] for x in turns[name]],
-                                    "frac_peak": tfv / MFMA_BF16_PEAK_TFLOPS, "peak_TFLOP/s": MFMA_BF16_PEAK_TFLOPS,
-                                    "what": "torch.mm (hipBLASLt), %s output; comparison only" % ("bf16" if name.endswith("bf16_out") else "fp32")}
+        else:
+            calls = {"gemm_f32_4096_vendor": lambda: torch.mm(dA, dB, out=dC)}
+        peak = MFMA_BF16_PEAK_TFLOPS if variant == "bf16" else FP32_PEAK_TFLOPS
+        turns = {"ours": [t]}
+        for turn in range(2):
+            for name, call in calls.items():
+                try:
+                    turns.setdefault(name, []).append(measure(call, 5, steps_here, torch, gern_amd))
+                except Exception as e:  # a torch without out_dtype: say so, do not fail the benchmark
+                    vendor[name] = {"error": str(e)[:200]}
+            if turn == 0:
+                turns["ours"].append(measure(lambda: g(dA, dB, dC), 5, steps_here, torch, gern_amd))
+        t = min(turns["ours"], key=lambda x: x["ms"])
+        for name in calls:
+            if name in turns:
+                tv = min(turns[name], key=lambda x: x["ms"])
+                tfv = 2.0 * n ** 3 / (tv["ms"] * 1e-3) / 1e12
+                vendor[name] = {"TFLOP/s": tfv, "ms": tv["ms"], "ms_median": tv["ms_median"], "ms_min": tv["ms_min"],
+                                "ms_turns": [x["ms"] for x in turns[name]],
+                                "frac_peak": tfv / peak, "peak_TFLOP/s": peak,
+                                "what": "torch.mm (hipBLASLt), %s operands, %s output; comparison only"
+                                        % (variant if variant == "bf16" else "fp32", "bf16" if name.endswith("bf16_out") else "fp32")}
         roof = roofline("gemm_%s_4096" % variant, table, bound, 2.0 * n ** 3, t, g)
         workloads["gemm_%s_4096" % variant] = {"TFLOP/s": roof["achieved"], "ms": t["ms"], "frac_peak": roof["frac"],
                                                "peak_TFLOP/s": roof["peak"], "roofline": roof}
         log("gemm %s 4096^3: %.1f us  %.1f TFLOP/s (%.1f%% of %.0f)" % (variant, t["ms"] * 1e3, roof["achieved"], 100 * roof["frac"], roof["peak"]))
-        if variant == "bf16":
-            workloads["gemm_bf16_4096"]["ms_turns"] = [x["ms"] for x in turns["ours"]]
-            workloads.update(vendor)
-            for name, v in vendor.items():
-                if "ms" in v:
-                    log("%s: %.1f us  %.1f TFLOP/s (turns: %s)" % (name, v["ms"] * 1e3, v["TFLOP/s"], ", ".join("%.1f" % (x * 1e3) for x in v["ms_turns"])))
+        workloads["gemm_%s_4096" % variant]["ms_turns"] = [x["ms"] for x in turns["ours"]]
+        workloads.update(vendor)
+        for name, v in vendor.items():
+            if "ms" in v:
+                log("%s: %.1f us  %.1f TFLOP/s (turns: %s)" % (name, v["ms"] * 1e3, v["TFLOP/s"], ", ".join("%.1f" % (x * 1e3) for x in v["ms_turns"])))
         if variant == "f32" and not args.no_cpu:
             from oracle import oracle as o
             from oracle import ref
