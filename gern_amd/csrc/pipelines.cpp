@@ -608,7 +608,21 @@ int gern_qk_softmax_create(int64_t head_dim, int64_t max_keys, int flags, gern_p
                 // block as it gets wider.
                 {{Grid::BLOCK_DIM_X, threads.bind(64 * qkWaves(max_keys))}});
         }
-        int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
+        // Tile kernel, rows of up to 4096 keys: XCD x takes row blocks x, x + 8, ... (bands of one row of tiles
+        // dealt to the XCDs in turn), so the sixteen workgroups that exchange a row block's statistics and write
+        // its rows sit on one XCD: 20.9 instead of 21.4-21.8 us at 4096 x 4096 x 128, same results.  A row block's
+        // workgroups then lie within 8 x 16 = 128 consecutive launch numbers instead of 16, and that many must be
+        // resident together for them to meet: taken only on a GPU with at least 256 CUs (one workgroup per CU), and
+        // not for wider rows, whose row blocks would lie 8 x N / 256 launch numbers apart.
+        bool rows_on_one_xcd = p->qk_tiles && max_keys <= 4096 && !(flags & GERN_PIPELINE_NO_XCD_REMAP);
+        if (rows_on_one_xcd && !(flags & GERN_PIPELINE_COMPILE_ONLY)) {
+            gern_hip_limits limits;
+            rows_on_one_xcd = gern_hip_device_limits(&limits) == 0 && limits.compute_units >= 256;
+        }
+        if (experiments() && std::getenv("GERN_QK_PLAIN_ORDER") != nullptr) {
+            rows_on_one_xcd = false;
+        }
+        int rc = rows_on_one_xcd ? finish(p.get(), program, flags, 0, 1) : finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
         if (rc != 0) {
             return rc;
         }

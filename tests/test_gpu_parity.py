@@ -649,6 +649,33 @@ def test_qk_softmax_tile_kernel_on_rows_wider_than_4096_keys(gpu, oracle, M, N, 
             gpu.QKSoftmax(96, 8192)  # the row-block kernel keeps whole rows in registers
 
 
+@pytest.mark.parametrize("M,N", [(4096, 4096), (8192, 4096), (300, 2560), (2100, 1000)])
+def test_qk_softmax_tile_kernel_either_workgroup_order_gives_the_same_bits(gpu, oracle, M, N):
+    # Rows of up to 4096 keys: by default every row block's tiles run on one XCD (XCD x takes row blocks x, x + 8,
+    # ...; launch numbers past the last whole group of eight row blocks keep their tiles); with NO_XCD_REMAP tiles
+    # are taken in launch order.  Which workgroup computes a tile changes nothing in it.
+    import torch
+    D = 128
+    qb, _ = oracle.to_bf16(oracle.normal((M, D), 81))
+    kb, _ = oracle.to_bf16(oracle.normal((N, D), 82))
+    scale = np.float32(1.0 / np.sqrt(D))
+    by_rows, in_order = gpu.QKSoftmax(D, 4096), gpu.QKSoftmax(D, 4096, flags=gpu.NO_XCD_REMAP)
+    assert "gern_band" in by_rows.source and "gern_band" not in in_order.source
+    results = []
+    for p in (by_rows, in_order):
+        S = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        p(_dev(qb.view(np.int16)), _dev(kb.view(np.int16)), S, scale)
+        torch.cuda.synchronize()
+        assert p.faults() == 0
+        results.append(S.cpu().numpy())
+    assert np.array_equal(results[0], results[1])
+    rows = sorted({0, 255, 256, M // 2, M - 1})
+    want = oracle.qk_softmax(qb[rows], kb, scale)
+    assert np.max(np.abs(results[0][rows] - want) / want) < 1e-2
+    # wider rows keep the launch order: their row blocks would lie too many launch numbers apart
+    assert "gern_band" not in gpu.QKSoftmax(D, 8192).source
+
+
 def test_qk_softmax_tile_kernel_over_changing_shapes_and_scales(gpu, oracle):
     # One pipeline, one exchange memory: every launch tags its entries with its
     # own number, so shapes may change from run to run (entries left by a wider
