@@ -6,6 +6,7 @@
 // test/test-nodes.cpp, test-same-expr.cpp, test-functions.cpp,
 // test-pipeline.cpp, test-grid-constraints.cpp, test-map-grid.cpp,
 // test-set-unit.cpp.
+#include "resolve_constraints/resolve_constraints.h"
 #include "annotations/data_dependency_language.h"
 #include "annotations/visitor.h"
 #include "compose/composable.h"
@@ -130,6 +131,49 @@ CASE("same_expr.compound") {  // test-same-expr.cpp:43-67
     REQUIRE(!isSameExpr(a + b * c, a - b * c));
     REQUIRE(!isSameExpr(a + b * c, a - b));
     REQUIRE(!isSameExpr(a + b * c, a));
+}
+
+// ---- test-resolve-constraints.cpp ------------------------------------------------
+// The reference's cases (its solver is GiNaC, whose answers come out over the rationals: y*0.25; here the
+// solution stays over the nodes of the equation: y / 4), and what the interface excludes.
+
+CASE("resolve.one_variable_on_either_side") {  // test-resolve-constraints.cpp:8-22
+    Variable x("x"), y("y");
+    Expr sol = resolve::solve(x == y, x);
+    REQUIRE(sol.ptr == y.ptr);  // the variable itself, as the reference asserts
+    REQUIRE_EQ(resolve::solve((x - 1) == y, x).str(), std::string("(y + 1)"));
+    REQUIRE_EQ(resolve::solve(x == y - 1, x).str(), std::string("(y - 1)"));
+    REQUIRE_EQ(resolve::solve(y == x + 3, x).str(), std::string("(y - 3)"));
+    REQUIRE_EQ(resolve::solve(Expr(7) == x, x).str(), std::string("7"));
+}
+
+CASE("resolve.coefficients") {  // test-resolve-constraints.cpp:24-36
+    Variable x("x"), y("y"), z("z");
+    REQUIRE_EQ(resolve::solve((x * 4) == y, x).str(), std::string("(y / 4)"));
+    REQUIRE(isSameExpr(resolve::solve(x * z == y, x), y / z));
+    REQUIRE(isSameExpr(resolve::solve(z * x == y, x), y / z));
+    REQUIRE_EQ(resolve::solve(x / 2 == y, x).str(), std::string("(y / 0.5)"));  // 1 / 2 is not a whole number: folded as a fraction
+    // literals fold: 2 x + 3 x = 10
+    REQUIRE_EQ(resolve::solve(x * 2 + x * 3 == Expr(10), x).str(), std::string("2"));
+}
+
+CASE("resolve.coefficients_and_sums") {  // test-resolve-constraints.cpp:38-47
+    Variable x("x"), y("y"), z("z");
+    REQUIRE_EQ(resolve::solve((x * 4) + z == y, x).str(), std::string("((y - z) / 4)"));
+    // the variable on both sides: 3 x + y = x + z
+    REQUIRE_EQ(resolve::solve(x * 3 + y == x + z, x).str(), std::string("((z - y) / 2)"));
+    // a tile's extent from its consumer's: l + stride - 1 = n
+    Variable l("l"), stride("stride"), n("n");
+    REQUIRE_EQ(resolve::solve(l + stride - 1 == n, l).str(), std::string("(n - (stride - 1))"));
+}
+
+CASE("resolve.what_is_not_linear_is_refused") {
+    Variable x("x"), y("y");
+    REQUIRE_THROWS_AS(resolve::solve(x * x == y, x), error::UserError);
+    REQUIRE_THROWS_AS(resolve::solve(y / x == Expr(2), x), error::UserError);
+    REQUIRE_THROWS_AS(resolve::solve(x % 4 == y, x), error::UserError);
+    REQUIRE_THROWS_AS(resolve::solve(y == Expr(3), x), error::UserError);   // x does not occur
+    REQUIRE_THROWS_AS(resolve::solve(x + y == x + 1, x), error::UserError);  // its coefficient cancels
 }
 
 // ---- test-functions.cpp -------------------------------------------------------
