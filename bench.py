@@ -178,7 +178,7 @@ extern "C" __global__ void __launch_bounds__(256) gern_copy_f4_streaming(const g
 """
 
 
-def copy_calibration(torch, gern_amd, warmup, steps, kernel="gern_copy_f4", nbytes=256 << 20):
+def copy_calibration(torch, gern_amd, warmup, steps, kernel="gern_copy_f4", nbytes=256 << 20, pairs=1):
     """A plain float4 copy of 256 MiB through the same C ABI.  gern_copy_f4 is
     the kernel of known size that the FETCH_SIZE / WRITE_SIZE counters are
     scaled by; gern_copy_f4_streaming (nontemporal stores, as the gernels use)
@@ -190,22 +190,31 @@ def copy_calibration(torch, gern_amd, warmup, steps, kernel="gern_copy_f4", nbyt
     if hip.gern_hip_compile(COPY_SRC.encode(), names, 1, None, 0, None, C.byref(mod)) != 0 or \
        hip.gern_hip_get_kernel(mod, kernel.encode(), C.byref(ker)) != 0:
         raise gern_amd.GernError(gern_amd._hip_error())
-    src = torch.ones(nbytes // 4, device="cuda")
-    dst = torch.zeros_like(src)
+    # pairs > 1: the launches go round that many buffer pairs, as the rotating-buffer runs of the pipelines do
+    srcs = [torch.ones(nbytes // 4, device="cuda") for _ in range(pairs)]
+    dsts = [torch.zeros_like(srcs[0]) for _ in range(pairs)]
     n = C.c_longlong(nbytes // 16)
-    a, b = C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())
-    params = (C.c_void_p * 3)(C.cast(C.byref(a), C.c_void_p), C.cast(C.byref(b), C.c_void_p), C.cast(C.byref(n), C.c_void_p))
     grid = (C.c_uint32 * 3)((nbytes // 16 + 255) // 256, 1, 1)
     block = (C.c_uint32 * 3)(256, 1, 1)
+    args_of = []
+    for src, dst in zip(srcs, dsts):
+        a, b = C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())
+        args_of.append((a, b, (C.c_void_p * 3)(C.cast(C.byref(a), C.c_void_p), C.cast(C.byref(b), C.c_void_p), C.cast(C.byref(n), C.c_void_p))))
+    turn = [0]
 
     def launch():
+        params = args_of[turn[0] % pairs][2]
+        turn[0] += 1
         if hip.gern_hip_launch(ker, grid, block, 0, params, None) != 0:
             raise gern_amd.GernError(gern_amd._hip_error())
     device_warmup(launch, torch)
     wall, ev = time_launches(launch, warmup, steps, torch, gern_amd)
-    assert bool((dst == 1).all())
-    return {"GB/s": 2 * nbytes / (ev * 1e-3) / 1e9, "ms": ev, "frac_hbm": 2 * nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "kernel": kernel, "bytes_read": nbytes, "bytes_written": nbytes}
+    assert all(bool((dst == 1).all()) for dst in dsts)
+    out = {"GB/s": 2 * nbytes / (ev * 1e-3) / 1e9, "ms": ev, "frac_hbm": 2 * nbytes / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "kernel": kernel, "bytes_read": nbytes, "bytes_written": nbytes}
+    if pairs > 1:
+        out["buffer_pairs"] = pairs
+    return out
 
 
 def cpu_blur(img_np, pattern, tile_rows, tile_cols, budget_s, what_size):
@@ -570,6 +579,12 @@ def main():
         log("copy 256 MiB, streaming stores: %.1f us  %.0f GB/s" % (workloads["copy_256MiB_streaming_stores"]["ms"] * 1e3,
                                                                    workloads["copy_256MiB_streaming_stores"]["GB/s"]))
         if not args.no_rotating:
+            # the blur's bytes in the blur's regime: 256 MiB in, 256 MiB out, round four buffer pairs
+            workloads["copy_256MiB_streaming_stores_rotating_buffers"] = copy_calibration(
+                torch, gern_amd, args.warmup, steps2, "gern_copy_f4_streaming", pairs=4)
+            log("copy 256 MiB, streaming stores, over 4 rotating buffer pairs: %.1f us  %.0f GB/s" % (
+                workloads["copy_256MiB_streaming_stores_rotating_buffers"]["ms"] * 1e3,
+                workloads["copy_256MiB_streaming_stores_rotating_buffers"]["GB/s"]))
             # 1 GiB: far beyond the 256 MiB memory-side cache, i.e. what HBM itself streams
             workloads["copy_1GiB_streaming_stores"] = copy_calibration(torch, gern_amd, args.warmup, max(10, steps2 // 2),
                                                                        "gern_copy_f4_streaming", 1 << 30)
