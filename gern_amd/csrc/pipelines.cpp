@@ -341,7 +341,9 @@ int gern_softmax_create(int64_t ncol, int64_t rows_per_wave, int flags, gern_pip
                                                               div(row_sum, expd, output))),
                    {{Grid::BLOCK_DIM_X, threads.bind(Grid::kWavefrontSize * waves)}});
         // Rows are contiguous and independent: plain launch order already
-        // streams through memory, and measures faster than the XCD order.
+        // streams through memory, and measures faster than the XCD order
+        // (8192 x 4096 over rotating buffers: 45.3 us; bands of 4, 16, 64, 256
+        // rows dealt to the XCDs in turn 46.3, 45.7, 46.9, 47.9 us).
         int rc = finish(p.get(), program, flags | GERN_PIPELINE_NO_XCD_REMAP);
         if (rc != 0) {
             return rc;
